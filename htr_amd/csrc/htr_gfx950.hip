@@ -1,0 +1,560 @@
+// HTR-W1 packed-linear kernels for MI355X (gfx950, CDNA4, wave64) behind a plain C ABI.
+//
+//   y = sv . Ho( Q . Hi(su . x) ),   Q[i,j] = v(s_ij) * scale_i * CBSCALE,
+//   v(s) = bytesum((s * 0xDF6ADF + 0x34983) mod 2^32) - 510              (docs/FORMAT.md:7-13 of the reference)
+//
+// Work decomposition of the fused linear kernel
+//   workgroup = 8 waves = one 128-row output block (one H128 output block) x one split of the input columns
+//   wave      = one 16-row strip of tiles; per step it streams the 8 consecutive tiles that cover one 128-column
+//               input block (8 * 32K contiguous bytes: each lane loads its 4K contiguous bytes)
+//   lane      = (tile-in-step = lane / 8, row pair q = lane % 8): the K dwords a lane loads are exactly the stream
+//               bits of tile rows 2q and 2q+1 (32 steps); the 16-K history bits come from the previous lane's last
+//               dword through the LDS crossbar (ds_bpermute), the tail-biting wrap is lane 7 -> lane 0 of the tile
+//   decode    = per weight: one bit-field extract, one v_mad_u32_u24, one v_sad_u8 / v_sad_hi_u8.  The SAD pair
+//               accumulates onto 0x64006400, which leaves two IEEE half floats 1024 + bytesum = 1534 + v packed in
+//               one dword with no integer->float conversion and no pack instruction.
+//   product   = v_mfma_f32_16x16x32_f16.  MFMA row i = lane % 16 = (tile parity h = i / 8, row pair q = i % 8), the
+//               four 16-lane groups g supply the k-slots, so lane (g, h, q) feeds tile 2g + h.  Rows with h = 0 and
+//               h = 1 need different activation columns; the B operand therefore carries, for activation row r,
+//               the even tiles in MFMA column 2r and the odd tiles in column 2r + 1, and only D[i][2r + h(i)] is
+//               kept.  Eight activation rows share one MFMA; more rows reuse the decoded A registers.
+//   offset    = the constant 1534 is removed afterwards with 1534 * sum(x~) per activation row.
+//   epilogue  = split partials meet in a workspace; the last workgroup of a row block (arrival counter) sums them in
+//               a fixed order, applies scale * CBSCALE, the output H128, sv, bias and the cast.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <string.h>
+
+#include "../../include/htr_gfx950.h"
+
+namespace {
+
+constexpr uint32_t GEN_A = 0xDF6ADFu;
+constexpr uint32_t GEN_B = 0x34983u;
+constexpr float INV_SQRT128 = 0.08838834764831845f;
+constexpr float SQRT128 = 11.313708498984761f;
+// 1 / sqrt(mean v^2) over all 65536 states: sum v^2 = 1433042863 (htr/wire.py:28-30 of the reference)
+constexpr double MEAN_SQ = 1433042863.0 / 65536.0;
+
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef float f4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u2 __attribute__((ext_vector_type(2)));
+
+constexpr int WG_WAVES = 8;
+constexpr int WG_THREADS = WG_WAVES * 64;
+constexpr int LDS_BUDGET = 64 * 1024;
+
+// ------------------------------------------------------------------------------------------------ small helpers
+__device__ __forceinline__ float bf16_bits_to_float(uint16_t b) { return __uint_as_float((uint32_t)b << 16); }
+__device__ __forceinline__ float f16_bits_to_float(uint16_t b) { return (float)__builtin_bit_cast(_Float16, b); }
+__device__ __forceinline__ uint16_t float_to_bf16_bits(float f) {   // round to nearest even
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40u);
+  return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+}
+__device__ __forceinline__ float load_elem(const void* p, int dtype, size_t idx) {
+  if (dtype == HTR_BF16) return bf16_bits_to_float(((const uint16_t*)p)[idx]);
+  if (dtype == HTR_F16) return f16_bits_to_float(((const uint16_t*)p)[idx]);
+  return ((const float*)p)[idx];
+}
+__device__ __forceinline__ void store_elem(void* p, int dtype, size_t idx, float v) {
+  if (dtype == HTR_BF16) ((uint16_t*)p)[idx] = float_to_bf16_bits(v);
+  else if (dtype == HTR_F16) ((uint16_t*)p)[idx] = __builtin_bit_cast(uint16_t, (_Float16)v);
+  else ((float*)p)[idx] = v;
+}
+__device__ __forceinline__ float sign_of(const uint8_t* bits, int j) { return ((bits[j >> 3] >> (j & 7)) & 1) ? -1.f : 1.f; }
+__device__ __forceinline__ float lane_xor(float v, int mask) { return __shfl_xor(v, mask, 64); }
+
+// 128-point Walsh-Hadamard butterfly network over one wave: lane holds elements `lane` (a) and `lane + 64` (b).
+__device__ __forceinline__ void fwht128_wave(float& a, float& b, int lane) {
+  float t = a + b; b = a - b; a = t;
+#pragma unroll
+  for (int h = 32; h >= 1; h >>= 1) {
+    const float pa = lane_xor(a, h), pb = lane_xor(b, h);
+    const bool up = (lane & h) != 0;
+    a = up ? (pa - a) : (a + pa);
+    b = up ? (pb - b) : (b + pb);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ stream loads
+// The K dwords of lane `lane` start at dword lane*K of the wave's 64*K-dword step: contiguous across the wave.
+template <int K> struct StreamRegs { uint32_t d[K]; };
+
+template <int K> __device__ __forceinline__ void load_stream(const uint32_t* __restrict__ p, StreamRegs<K>& r) {
+  if constexpr (K == 2) {
+    u2 v = __builtin_nontemporal_load((const u2*)p); r.d[0] = v.x; r.d[1] = v.y;
+  } else if constexpr (K == 4) {
+    u4 v = __builtin_nontemporal_load((const u4*)p); r.d[0] = v.x; r.d[1] = v.y; r.d[2] = v.z; r.d[3] = v.w;
+  } else if constexpr (K == 8) {
+    u4 v = __builtin_nontemporal_load((const u4*)p), w = __builtin_nontemporal_load((const u4*)p + 1);
+    r.d[0] = v.x; r.d[1] = v.y; r.d[2] = v.z; r.d[3] = v.w; r.d[4] = w.x; r.d[5] = w.y; r.d[6] = w.z; r.d[7] = w.w;
+  } else if constexpr (K == 6) {
+    const u2* q = (const u2*)p;
+    u2 a = __builtin_nontemporal_load(q), b = __builtin_nontemporal_load(q + 1), c = __builtin_nontemporal_load(q + 2);
+    r.d[0] = a.x; r.d[1] = a.y; r.d[2] = b.x; r.d[3] = b.y; r.d[4] = c.x; r.d[5] = c.y;
+  } else {
+#pragma unroll
+    for (int k = 0; k < K; ++k) r.d[k] = __builtin_nontemporal_load(p + k);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ decode core
+// V[0] = the dword before the lane's first dword (history), V[1..K] = the lane's dwords.  Local step u (0..31) is
+// trellis step t = 32q + u; its state is the 16 bits of V that start at bit 16 + (u + 1) * K (bit 0 = MSB of V[0]).
+template <int K> struct Window {
+  uint32_t V[K + 1];
+  uint32_t mid[K];     // mid[w] = bits [32w + 16, 32w + 48) of V, for windows that straddle two dwords
+  __device__ __forceinline__ void build(const StreamRegs<K>& r, uint32_t prev) {
+    V[0] = prev;
+#pragma unroll
+    for (int k = 0; k < K; ++k) V[k + 1] = r.d[k];
+#pragma unroll
+    for (int k = 0; k < K; ++k) mid[k] = __builtin_amdgcn_alignbit(V[k], V[k + 1], 16);
+  }
+  template <int U> __device__ __forceinline__ uint32_t state() const {
+    constexpr int b = 16 + (U + 1) * K, w = b >> 5, off = b & 31;
+    if constexpr (off <= 16) return (V[w] >> (16 - off)) & 0xFFFFu;
+    else return (mid[w] >> (32 - off)) & 0xFFFFu;
+  }
+  // generator word x = s*A + B; s < 2^16 and A < 2^24 so this is one v_mad_u32_u24
+  template <int U> __device__ __forceinline__ uint32_t genword() const { return state<U>() * GEN_A + GEN_B; }
+  // two consecutive weights as packed halves (1534 + v(u), 1534 + v(u + 1))
+  template <int U> __device__ __forceinline__ uint32_t pair_f16() const {
+    uint32_t r = __builtin_amdgcn_sad_u8(genword<U>(), 0u, 0x64006400u);
+    return __builtin_amdgcn_sad_hi_u8(genword<U + 1>(), 0u, r);
+  }
+  template <int U> __device__ __forceinline__ int value() const {   // integer v(s)
+    return (int)__builtin_amdgcn_sad_u8(genword<U>(), 0u, 0u) - 510;
+  }
+  template <int U0> __device__ __forceinline__ h8 group8() const {   // 8 consecutive weights as an MFMA operand
+    u4 v = {pair_f16<U0>(), pair_f16<U0 + 2>(), pair_f16<U0 + 4>(), pair_f16<U0 + 6>()};
+    return __builtin_bit_cast(h8, v);
+  }
+};
+
+// lane that holds the dword preceding this lane's first dword: previous row pair of the same tile, circular
+__device__ __forceinline__ int history_lane_byteaddr(int lane) { return ((lane & ~7) | ((lane - 1) & 7)) << 2; }
+
+// ------------------------------------------------------------------------------------------------ fused linear
+struct LinearArgs {
+  const uint32_t* qw;
+  const uint16_t* scales;
+  const uint8_t* su;
+  const uint8_t* sv;
+  const void* x;
+  const void* bias;
+  void* y;
+  float* part;
+  uint32_t* cnt;
+  int m, n, M, ns, bps, x_dtype, y_dtype;
+  float cbscale;
+};
+
+// LDS layout (dynamic): [xt: (M + 1) rows x row_halves f16][amax: 32 u32][sc: 32 f32][xs: M * bps f32][yt: M * 128 f32]
+__host__ __device__ inline int xt_row_halves(int bps) { return bps * 128 + 8; }   // +8 halves: rows land on different banks
+__host__ __device__ inline size_t lds_bytes(int M, int bps) {
+  return (size_t)(M + 1) * xt_row_halves(bps) * 2 + 32 * 4 + 32 * 4 + (size_t)M * bps * 4 + (size_t)M * 128 * 4;
+}
+
+template <int K, int MB, int P>
+__global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
+  extern __shared__ __align__(16) unsigned char lds[];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int rb = blockIdx.x / a.ns, sp = blockIdx.x - rb * a.ns;
+  const int nblk = a.n >> 7, nt = a.n >> 4;
+  const int b0 = sp * a.bps, nb = min(nblk, b0 + a.bps) - b0;
+  const int M = a.M;
+  const int rowh = xt_row_halves(a.bps);
+
+  _Float16* xt = (_Float16*)lds;
+  uint32_t* s_amax = (uint32_t*)(lds + (size_t)(M + 1) * rowh * 2);
+  float* s_sc = (float*)(s_amax + 32);
+  float* s_xs = s_sc + 32;
+  float* s_y = s_xs + M * a.bps;
+
+  // ---- start the weight stream first: everything below overlaps with these loads
+  const uint32_t* wp = a.qw + ((size_t)(rb * 8 + w) * nt + (size_t)8 * b0) * (8 * K) + lane * K;
+  constexpr int STEP_DWORDS = 64 * K;
+  StreamRegs<K> buf[P];
+#pragma unroll
+  for (int p = 0; p < P; ++p)
+    if (p < nb) load_stream<K>(wp + (size_t)p * STEP_DWORDS, buf[p]);
+
+  // ---- input rotation of this split's columns: x~ = f16( H128(su . x) / sqrt(128) / sc ), sc a power of two per row
+  if (threadIdx.x < 32) s_amax[threadIdx.x] = 0u;
+  for (int i = threadIdx.x; i < rowh / 2; i += WG_THREADS) ((uint32_t*)(xt + (size_t)M * rowh))[i] = 0u;   // zero row
+  __syncthreads();
+  const int npairs = M * nb;
+  for (int pi = w; pi < npairs; pi += WG_WAVES) {
+    const int mrow = pi / nb, bl = pi - mrow * nb;
+    const size_t base = (size_t)mrow * a.n + (size_t)(b0 + bl) * 128;
+    float mx = fmaxf(fabsf(load_elem(a.x, a.x_dtype, base + lane)), fabsf(load_elem(a.x, a.x_dtype, base + lane + 64)));
+#pragma unroll
+    for (int h = 32; h >= 1; h >>= 1) mx = fmaxf(mx, lane_xor(mx, h));
+    if (lane == 0) atomicMax(&s_amax[mrow], __float_as_uint(mx));
+  }
+  __syncthreads();
+  for (int pi = w; pi < npairs; pi += WG_WAVES) {
+    const int mrow = pi / nb, bl = pi - mrow * nb;
+    const int col = (b0 + bl) * 128;
+    const size_t base = (size_t)mrow * a.n + col;
+    // |H128 x| / sqrt(128) <= sqrt(128) * amax; keep that bound in (8192, 16384] so f16 neither overflows nor
+    // loses small activations to denormals
+    const float bound = __uint_as_float(s_amax[mrow]) * SQRT128;
+    int e = 0;
+    if (bound > 0.f && bound < 3.0e38f) e = ilogbf(bound) - 13;
+    const float inv_sc = ldexpf(1.f, -e);
+    float va = load_elem(a.x, a.x_dtype, base + lane) * sign_of(a.su, col + lane) * inv_sc;
+    float vb = load_elem(a.x, a.x_dtype, base + lane + 64) * sign_of(a.su, col + lane + 64) * inv_sc;
+    fwht128_wave(va, vb, lane);
+    const _Float16 ha = (_Float16)(va * INV_SQRT128), hb = (_Float16)(vb * INV_SQRT128);
+    xt[(size_t)mrow * rowh + bl * 128 + lane] = ha;
+    xt[(size_t)mrow * rowh + bl * 128 + lane + 64] = hb;
+    float s = (float)ha + (float)hb;
+#pragma unroll
+    for (int h = 32; h >= 1; h >>= 1) s += lane_xor(s, h);
+    if (lane == 0) {
+      s_xs[pi] = s;
+      if (bl == 0) s_sc[mrow] = ldexpf(1.f, e);
+    }
+  }
+  __syncthreads();
+
+  // ---- main loop: one 128-column block (8 tiles of this wave's strip) per step
+  const int g = lane >> 4, n16 = lane & 15;
+  int boff[MB];   // LDS half-index of this lane's B operand for the first block of the split
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    const int mrow = mb * 8 + (n16 >> 1);
+    boff[mb] = (mrow < M ? mrow : M) * rowh + 16 * (2 * g + (n16 & 1));
+  }
+  const int hist = history_lane_byteaddr(lane);
+  f4 acc[MB][2];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) { acc[mb][0] = f4{0.f, 0.f, 0.f, 0.f}; acc[mb][1] = f4{0.f, 0.f, 0.f, 0.f}; }
+
+  for (int s0 = 0; s0 < nb; s0 += P) {
+#pragma unroll
+    for (int p = 0; p < P; ++p) {
+      const int s = s0 + p;
+      if (s < nb) {
+        const StreamRegs<K> cur = buf[p];
+        if (s + P < nb) load_stream<K>(wp + (size_t)(s + P) * STEP_DWORDS, buf[p]);
+        Window<K> win;
+        win.build(cur, (uint32_t)__builtin_amdgcn_ds_bpermute(hist, (int)cur.d[K - 1]));
+        h8 B0[MB], B1[MB];
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+          const _Float16* bp = xt + boff[mb] + s * 128;
+          B0[mb] = *(const h8*)bp;
+          B1[mb] = *(const h8*)(bp + 8);
+        }
+        const h8 A0 = win.template group8<0>();     // row 2q,     columns 0..7 of the lane's tile
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) acc[mb][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A0, B0[mb], acc[mb][0], 0, 0, 0);
+        const h8 A1 = win.template group8<8>();     // row 2q,     columns 8..15
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) acc[mb][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A1, B1[mb], acc[mb][0], 0, 0, 0);
+        const h8 A2 = win.template group8<16>();    // row 2q + 1, columns 0..7
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) acc[mb][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A2, B0[mb], acc[mb][1], 0, 0, 0);
+        const h8 A3 = win.template group8<24>();    // row 2q + 1, columns 8..15
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) acc[mb][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A3, B1[mb], acc[mb][1], 0, 0, 0);
+      }
+    }
+  }
+
+  // ---- fold the two tile parities, remove the 1534 offset, undo the activation scale -> this split's partial
+  // D[i][c] sits in lane c + 16 * (i / 4), register i % 4.  Row pair q is D row q (even tiles, column 2r) plus
+  // D row q + 8 (odd tiles, column 2r + 1): lane (g', c) with g' < 2 and c even adds lane + 33.
+  {
+    const int partner = ((lane + 33) & 63) << 2;
+    const bool keeper = g < 2 && (n16 & 1) == 0;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      const int mrow = mb * 8 + (n16 >> 1);
+      float xs = 0.f, sc = 0.f;
+      if (keeper && mrow < M) {
+        for (int bl = 0; bl < nb; ++bl) xs += s_xs[mrow * nb + bl];
+        sc = s_sc[mrow];
+      }
+#pragma unroll
+      for (int rr = 0; rr < 2; ++rr)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const float mine = acc[mb][rr][j];
+          const float other = __uint_as_float((uint32_t)__builtin_amdgcn_ds_bpermute(partner, (int)__float_as_uint(mine)));
+          if (keeper && mrow < M) s_y[mrow * 128 + 16 * w + 2 * (4 * g + j) + rr] = ((mine + other) - 1534.f * xs) * sc;
+        }
+    }
+  }
+  __syncthreads();
+
+  if (a.ns > 1) {
+    float* mypart = a.part + ((size_t)(rb * a.ns + sp) * M) * 128;
+    for (int i = threadIdx.x; i < M * 128; i += WG_THREADS) mypart[i] = s_y[i];
+    __threadfence();
+    __syncthreads();
+    __shared__ int s_last;
+    if (threadIdx.x == 0) s_last = (atomicAdd(&a.cnt[rb], 1u) == (uint32_t)(a.ns - 1));
+    __syncthreads();
+    if (!s_last) return;
+    __threadfence();
+  }
+
+  // ---- output side: sum the splits in a fixed order, row scale, H128, sv, bias, cast
+  for (int mrow = w; mrow < M; mrow += WG_WAVES) {
+    float v0, v1;
+    if (a.ns > 1) {
+      v0 = 0.f; v1 = 0.f;
+      const float* pp = a.part + ((size_t)rb * a.ns * M + mrow) * 128;
+      for (int s = 0; s < a.ns; ++s) {
+        v0 += __builtin_nontemporal_load(pp + (size_t)s * M * 128 + lane);
+        v1 += __builtin_nontemporal_load(pp + (size_t)s * M * 128 + lane + 64);
+      }
+    } else {
+      v0 = s_y[mrow * 128 + lane];
+      v1 = s_y[mrow * 128 + lane + 64];
+    }
+    const int r0 = rb * 128 + lane, r1 = r0 + 64;
+    v0 *= f16_bits_to_float(a.scales[r0]) * a.cbscale;
+    v1 *= f16_bits_to_float(a.scales[r1]) * a.cbscale;
+    fwht128_wave(v0, v1, lane);
+    v0 = v0 * INV_SQRT128 * sign_of(a.sv, r0);
+    v1 = v1 * INV_SQRT128 * sign_of(a.sv, r1);
+    if (a.bias != nullptr) {
+      v0 += load_elem(a.bias, a.y_dtype, r0);
+      v1 += load_elem(a.bias, a.y_dtype, r1);
+    }
+    store_elem(a.y, a.y_dtype, (size_t)mrow * a.m + r0, v0);
+    store_elem(a.y, a.y_dtype, (size_t)mrow * a.m + r1, v1);
+  }
+  if (a.ns > 1 && threadIdx.x == 0) a.cnt[rb] = 0u;   // leave the counter ready for the next call
+}
+
+// ------------------------------------------------------------------------------------------------ debug decodes
+template <int K, int U> struct ForEach32 {
+  template <typename F> __device__ __forceinline__ static void run(const Window<K>& w, F&& f) {
+    f(U, w.template value<U>());
+    if constexpr (U + 1 < 32) ForEach32<K, U + 1>::run(w, f);
+  }
+};
+
+template <int K>
+__global__ __launch_bounds__(256) void k_decode_raw(const uint32_t* __restrict__ qw, int16_t* __restrict__ out, int64_t ntiles) {
+  // thread = (tile, row pair q); the 8 threads of a tile are consecutive lanes
+  const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int lane = threadIdx.x & 63;
+  const bool live = gid < ntiles * 8;
+  StreamRegs<K> r;
+#pragma unroll
+  for (int k = 0; k < K; ++k) r.d[k] = 0u;
+  if (live) load_stream<K>(qw + gid * K, r);
+  const uint32_t prev = (uint32_t)__builtin_amdgcn_ds_bpermute(history_lane_byteaddr(lane), (int)r.d[K - 1]);
+  if (!live) return;
+  Window<K> w;
+  w.build(r, prev);
+  int16_t vals[32];
+  ForEach32<K, 0>::run(w, [&](int u, int v) { vals[u] = (int16_t)v; });
+  u4* o = (u4*)(out + gid * 32);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    u4 pk;
+    pk.x = (uint16_t)vals[8 * i + 0] | ((uint32_t)(uint16_t)vals[8 * i + 1] << 16);
+    pk.y = (uint16_t)vals[8 * i + 2] | ((uint32_t)(uint16_t)vals[8 * i + 3] << 16);
+    pk.z = (uint16_t)vals[8 * i + 4] | ((uint32_t)(uint16_t)vals[8 * i + 5] << 16);
+    pk.w = (uint16_t)vals[8 * i + 6] | ((uint32_t)(uint16_t)vals[8 * i + 7] << 16);
+    o[i] = pk;
+  }
+}
+
+template <int K>
+__global__ __launch_bounds__(256) void k_dequant_q(const uint32_t* __restrict__ qw, const uint16_t* __restrict__ scales,
+                                                   float* __restrict__ Q, int mt, int nt, double rms) {
+  const int64_t gid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  const int lane = threadIdx.x & 63;
+  const int64_t ntiles = (int64_t)mt * nt;
+  const bool live = gid < ntiles * 8;
+  StreamRegs<K> r;
+#pragma unroll
+  for (int k = 0; k < K; ++k) r.d[k] = 0u;
+  if (live) load_stream<K>(qw + gid * K, r);
+  const uint32_t prev = (uint32_t)__builtin_amdgcn_ds_bpermute(history_lane_byteaddr(lane), (int)r.d[K - 1]);
+  if (!live) return;
+  Window<K> w;
+  w.build(r, prev);
+  const int64_t tile = gid >> 3;
+  const int q = (int)(gid & 7);
+  const int ti = (int)(tile / nt), tj = (int)(tile - (int64_t)ti * nt);
+  const int64_t n = (int64_t)nt * 16;
+  const int row0 = ti * 16 + 2 * q;
+  const float sc0 = f16_bits_to_float(scales[row0]), sc1 = f16_bits_to_float(scales[row0 + 1]);
+  float* o0 = Q + (int64_t)row0 * n + (int64_t)tj * 16;
+  float* o1 = o0 + n;
+  // cb[s] = float32(v / rms) with the division in float64, then one float32 multiply (htr/wire.py:24,102 of the reference)
+  ForEach32<K, 0>::run(w, [&](int u, int v) {
+    const float cb = (float)((double)v / rms);
+    if (u < 16) o0[u] = cb * sc0; else o1[u - 16] = cb * sc1;
+  });
+}
+
+// ------------------------------------------------------------------------------------------------ host side
+thread_local int g_last_hip_error = 0;
+
+struct Plan { int ns, bps, mb; size_t lds; };
+
+inline bool make_plan(int m, int n, int M, int nsplit, Plan& pl) {
+  const int nblk = n / 128, rbs = m / 128;
+  pl.mb = M <= 8 ? 1 : (M <= 16 ? 2 : 4);
+  // largest number of 128-column blocks per workgroup that fits the LDS budget
+  int bps_max = 1;
+  while (bps_max < nblk && lds_bytes(M, bps_max + 1) <= (size_t)LDS_BUDGET) ++bps_max;
+  int ns;
+  if (nsplit > 0) ns = nsplit;
+  else {
+    // enough workgroups for two per CU, but at least two column blocks each when the matrix allows
+    ns = (512 + rbs - 1) / rbs;
+    if (ns > nblk / 2) ns = nblk / 2;
+    if (ns < 1) ns = 1;
+  }
+  if (ns > nblk) ns = nblk;
+  int bps = (nblk + ns - 1) / ns;
+  if (bps > bps_max) { if (nsplit > 0) return false; bps = bps_max; }
+  ns = (nblk + bps - 1) / bps;
+  pl.ns = ns; pl.bps = bps; pl.lds = lds_bytes(M, bps);
+  return true;
+}
+
+inline size_t counters_bytes(int m) { return (((size_t)(m / 128) * 4) + 255) / 256 * 256; }
+
+template <int K, int MB> int launch_linear_kmb(const LinearArgs& a, int grid, size_t lds, hipStream_t st) {
+  constexpr int P = K <= 4 ? 4 : (K <= 6 ? 3 : 2);
+  auto kern = k_linear<K, MB, P>;
+  if (lds > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
+  }
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(WG_THREADS), lds, st, a);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
+  return HTR_OK;
+}
+template <int K> int launch_linear_k(const LinearArgs& a, int mb, int grid, size_t lds, hipStream_t st) {
+  switch (mb) {
+    case 1: return launch_linear_kmb<K, 1>(a, grid, lds, st);
+    case 2: return launch_linear_kmb<K, 2>(a, grid, lds, st);
+    default: return launch_linear_kmb<K, 4>(a, grid, lds, st);
+  }
+}
+
+#define HTR_FOR_K(K, EXPR)                 \
+  switch (K) {                             \
+    case 2: { constexpr int KK = 2; EXPR; } break; \
+    case 3: { constexpr int KK = 3; EXPR; } break; \
+    case 4: { constexpr int KK = 4; EXPR; } break; \
+    case 5: { constexpr int KK = 5; EXPR; } break; \
+    case 6: { constexpr int KK = 6; EXPR; } break; \
+    case 7: { constexpr int KK = 7; EXPR; } break; \
+    case 8: { constexpr int KK = 8; EXPR; } break; \
+    default: return HTR_ERR_K;             \
+  }
+
+inline bool dtype_ok(int d) { return d == HTR_BF16 || d == HTR_F16 || d == HTR_F32; }
+
+}  // namespace
+
+// ================================================================================================ C ABI
+extern "C" {
+
+const char* htr_strerror(int status) {
+  switch (status) {
+    case HTR_OK: return "ok";
+    case HTR_ERR_NULL: return "a required pointer is NULL";
+    case HTR_ERR_K: return "unsupported K (HTR-W1 allows 2..8)";
+    case HTR_ERR_SHAPE: return "m and n must be positive multiples of 128";
+    case HTR_ERR_BATCH: return "M must be in 1..32 for one launch";
+    case HTR_ERR_DTYPE: return "dtype must be bf16 (0), f16 (1) or f32 (2)";
+    case HTR_ERR_WORKSPACE: return "workspace too small or not 256-byte aligned";
+    case HTR_ERR_ALIGN: return "tensor pointer not aligned (qweight 16 B, others natural)";
+    case HTR_ERR_LAUNCH: return "HIP launch failed";
+    case HTR_ERR_SPLIT: return "explicit split count does not fit this shape";
+    case HTR_ERR_COUNT: return "problem count out of range";
+    default: return "unknown status";
+  }
+}
+
+int htr_last_hip_error(void) { return g_last_hip_error; }
+int htr_abi_version(void) { return 1; }
+float htr_cbscale(void) { return (float)(1.0 / __builtin_sqrt(MEAN_SQ)); }
+
+size_t htr_workspace_bytes(int m, int n, int K, int M, int nsplit) {
+  if (K < 2 || K > 8 || m <= 0 || n <= 0 || m % 128 || n % 128 || M < 1 || M > HTR_MAX_BATCH) return 0;
+  Plan pl;
+  if (!make_plan(m, n, M, nsplit, pl)) return 0;
+  size_t bytes = counters_bytes(m);
+  if (pl.ns > 1) bytes += (size_t)(m / 128) * pl.ns * M * 128 * sizeof(float);
+  return bytes;
+}
+
+int htr_linear(const void* qweight, const void* scales, const void* su, const void* sv, const void* x, const void* bias,
+               void* y, int m, int n, int K, int M, int x_dtype, int y_dtype, int nsplit, void* workspace,
+               size_t workspace_bytes, void* stream) {
+  if (!qweight || !scales || !su || !sv || !x || !y) return HTR_ERR_NULL;
+  if (K < 2 || K > 8) return HTR_ERR_K;
+  if (m <= 0 || n <= 0 || m % 128 || n % 128) return HTR_ERR_SHAPE;
+  if (M < 1 || M > HTR_MAX_BATCH) return HTR_ERR_BATCH;
+  if (!dtype_ok(x_dtype) || !dtype_ok(y_dtype)) return HTR_ERR_DTYPE;
+  if (((uintptr_t)qweight & 15) || ((uintptr_t)scales & 1) || ((uintptr_t)x & (x_dtype == HTR_F32 ? 3 : 1)) ||
+      ((uintptr_t)y & (y_dtype == HTR_F32 ? 3 : 1)) || (bias && ((uintptr_t)bias & (y_dtype == HTR_F32 ? 3 : 1))))
+    return HTR_ERR_ALIGN;
+  Plan pl;
+  if (!make_plan(m, n, M, nsplit, pl)) return HTR_ERR_SPLIT;
+  const size_t need = htr_workspace_bytes(m, n, K, M, nsplit);
+  if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255)) return HTR_ERR_WORKSPACE;
+
+  LinearArgs a;
+  a.qw = (const uint32_t*)qweight; a.scales = (const uint16_t*)scales; a.su = (const uint8_t*)su; a.sv = (const uint8_t*)sv;
+  a.x = x; a.bias = bias; a.y = y;
+  a.cnt = (uint32_t*)workspace;
+  a.part = (float*)((unsigned char*)workspace + counters_bytes(m));
+  a.m = m; a.n = n; a.M = M; a.ns = pl.ns; a.bps = pl.bps; a.x_dtype = x_dtype; a.y_dtype = y_dtype;
+  a.cbscale = htr_cbscale();
+  const int grid = (m / 128) * pl.ns;
+  hipStream_t st = (hipStream_t)stream;
+  HTR_FOR_K(K, return launch_linear_k<KK>(a, pl.mb, grid, pl.lds, st));
+  return HTR_OK;
+}
+
+int htr_decode_raw(const void* qweight, void* out_i16, int64_t ntiles, int K, void* stream) {
+  if (!qweight || !out_i16) return HTR_ERR_NULL;
+  if (K < 2 || K > 8) return HTR_ERR_K;
+  if (ntiles <= 0) return HTR_ERR_SHAPE;
+  if (((uintptr_t)qweight & 15) || ((uintptr_t)out_i16 & 15)) return HTR_ERR_ALIGN;
+  const int64_t blocks = (ntiles * 8 + 255) / 256;
+  hipStream_t st = (hipStream_t)stream;
+  HTR_FOR_K(K, hipLaunchKernelGGL(k_decode_raw<KK>, dim3((unsigned)blocks), dim3(256), 0, st, (const uint32_t*)qweight,
+                                  (int16_t*)out_i16, ntiles));
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
+  return HTR_OK;
+}
+
+int htr_dequant_q(const void* qweight, const void* scales, void* out_f32, int mt, int nt, int K, void* stream) {
+  if (!qweight || !scales || !out_f32) return HTR_ERR_NULL;
+  if (K < 2 || K > 8) return HTR_ERR_K;
+  if (mt <= 0 || nt <= 0) return HTR_ERR_SHAPE;
+  if (((uintptr_t)qweight & 15) || ((uintptr_t)out_f32 & 3) || ((uintptr_t)scales & 1)) return HTR_ERR_ALIGN;
+  const int64_t blocks = ((int64_t)mt * nt * 8 + 255) / 256;
+  hipStream_t st = (hipStream_t)stream;
+  const double rms = __builtin_sqrt(MEAN_SQ);
+  HTR_FOR_K(K, hipLaunchKernelGGL(k_dequant_q<KK>, dim3((unsigned)blocks), dim3(256), 0, st, (const uint32_t*)qweight,
+                                  (const uint16_t*)scales, (float*)out_f32, mt, nt, rms));
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
+  return HTR_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,128 @@
+"""Python entry points of the MI355X HTR-W1 packed-linear path + torch custom op htr::linear.
+
+Same surface as htr/ops.py of the reference (linear(), the custom op and its fake, the
+M-based dispatch of _linear_impl, htr/ops.py:69-122), but the body calls the gfx950 library
+through its C ABI: tensors are passed as raw device pointers together with the current
+torch stream; outputs and the workspace are allocated here with torch.
+"""
+import os
+
+import torch
+
+from . import _native, wire
+
+CB = wire.cbscale()
+_DTYPE_CODE = {torch.bfloat16: _native.BF16, torch.float16: _native.F16, torch.float32: _native.F32}
+
+# One launch takes up to this many activation rows; longer inputs are cut into chunks that each
+# re-read the packed weight (the reference does the same in 8-row chunks, htr/ops.py:77-88).
+LAUNCH_MAX_M = _native.MAX_BATCH
+# explicit column-split count for experiments; 0 = library policy
+NSPLIT = int(os.environ.get("HTR_NSPLIT", "0"))
+
+_WORKSPACES = {}
+
+
+def workspace(device, stream_id, nbytes):
+    """Zeroed scratch for split partials and arrival counters, one per (device, stream).
+
+    The reference keeps one counter tensor per device (htr/ops.py:24-28), which two streams
+    would corrupt; keying by stream keeps concurrent streams apart.  Kernels leave the
+    counter words zero, so the buffer is zeroed only when it is (re)allocated.
+    """
+    key = (device.index, stream_id)
+    ws = _WORKSPACES.get(key)
+    if ws is None or ws.numel() < nbytes:
+        size = max(int(nbytes), 1 << 20)
+        ws = torch.zeros(size, dtype=torch.uint8, device=device)
+        _WORKSPACES[key] = ws
+    return ws
+
+
+def _launch(x2, qweight, scales, su, sv, bias, y, m, n, K, out_code):
+    L = _native.lib()
+    M = x2.shape[0]
+    need = L.htr_workspace_bytes(m, n, K, M, NSPLIT)
+    if need == 0:
+        raise RuntimeError("libhtr_gfx950: no launch plan for this shape / split")
+    stream = torch.cuda.current_stream(x2.device)
+    ws = workspace(x2.device, stream.cuda_stream, need)
+    _native.check(L.htr_linear(qweight.data_ptr(), scales.data_ptr(), su.data_ptr(), sv.data_ptr(), x2.data_ptr(),
+                               None if bias is None else bias.data_ptr(), y.data_ptr(), m, n, K, M,
+                               _DTYPE_CODE[x2.dtype], out_code, NSPLIT, ws.data_ptr(), ws.numel(), stream.cuda_stream))
+
+
+def _linear_impl(x2, qweight, scales, su, sv, bias, out_dtype=None):
+    m, n, K = wire.check_shapes(qweight, scales, su, sv)
+    M = x2.shape[0]
+    if x2.dim() != 2 or x2.shape[1] != n:
+        raise RuntimeError(f"x has {x2.shape[-1]} input features, weight expects {n}")
+    if x2.dtype not in _DTYPE_CODE:
+        raise KeyError(x2.dtype)
+    out_dtype = x2.dtype if out_dtype is None else out_dtype
+    if M == 0:
+        return x2.new_empty((0, m), dtype=out_dtype)
+    if not x2.is_cuda:
+        raise RuntimeError("htr::linear runs on a ROCm device only; move the tensors to the GPU")
+    for t in (qweight, scales, su, sv):
+        if t.device != x2.device or not t.is_contiguous():
+            raise RuntimeError("HTR-W1 tensors must be contiguous and on the device of x")
+    if bias is not None and (bias.dtype != out_dtype or bias.numel() != m or bias.device != x2.device):
+        raise RuntimeError("bias must be [m] in the output dtype on the device of x")
+    y = torch.empty((M, m), dtype=out_dtype, device=x2.device)
+    code = _DTYPE_CODE[out_dtype]
+    with torch.cuda.device(x2.device):
+        for r0 in range(0, M, LAUNCH_MAX_M):
+            r1 = min(M, r0 + LAUNCH_MAX_M)
+            _launch(x2[r0:r1], qweight, scales, su, sv, bias, y[r0:r1], m, n, K, code)
+    return y
+
+
+@torch.library.custom_op("htr::linear", mutates_args=())
+def htr_linear_op(x2: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor, su: torch.Tensor, sv: torch.Tensor,
+                  bias: torch.Tensor | None) -> torch.Tensor:
+    return _linear_impl(x2.contiguous(), qweight, scales, su, sv, bias)
+
+
+@htr_linear_op.register_fake
+def _(x2, qweight, scales, su, sv, bias):
+    return x2.new_empty((x2.shape[0], qweight.shape[0] * 16))
+
+
+def linear(x, qweight, scales, su, sv, bias=None):
+    """y = x @ W^T (+bias) for an HTR-W1 weight. x [..., n] -> [..., m] in x.dtype."""
+    shp = x.shape
+    y = htr_linear_op(x.reshape(-1, shp[-1]), qweight, scales, su, sv, bias)
+    return y.reshape(*shp[:-1], qweight.shape[0] * 16)
+
+
+def linear_f32out(x, qweight, scales, su, sv, bias=None):
+    """Same product with a float32 result (bias, if given, must be float32).  Used by accuracy checks."""
+    shp = x.shape
+    y = _linear_impl(x.reshape(-1, shp[-1]).contiguous(), qweight, scales, su, sv, bias, out_dtype=torch.float32)
+    return y.reshape(*shp[:-1], qweight.shape[0] * 16)
+
+
+def decode_raw(qweight):
+    """int16 [ntiles, 256] of v(s) per weight in tile order (decode_raw of the reference extension)."""
+    K = wire.bits_of(qweight)
+    ntiles = qweight.numel() // (8 * K)
+    if not qweight.is_cuda or not qweight.is_contiguous() or qweight.dtype != torch.int32:
+        raise RuntimeError("decode_raw wants a contiguous int32 device tensor")
+    out = torch.empty((ntiles, 256), dtype=torch.int16, device=qweight.device)
+    with torch.cuda.device(qweight.device):
+        st = torch.cuda.current_stream(qweight.device).cuda_stream
+        _native.check(_native.lib().htr_decode_raw(qweight.data_ptr(), out.data_ptr(), ntiles, K, st))
+    return out
+
+
+def dequant_q(qweight, scales):
+    """Rotated-domain Q float32 [m, n], bit-exact with the reference CPU decoder (wire.dequant_Q)."""
+    mt, nt, W = qweight.shape
+    if not qweight.is_cuda or not qweight.is_contiguous() or scales.dtype != torch.float16:
+        raise RuntimeError("dequant_q wants contiguous device tensors (int32 qweight, float16 scales)")
+    out = torch.empty((mt * 16, nt * 16), dtype=torch.float32, device=qweight.device)
+    with torch.cuda.device(qweight.device):
+        st = torch.cuda.current_stream(qweight.device).cuda_stream
+        _native.check(_native.lib().htr_dequant_q(qweight.data_ptr(), scales.data_ptr(), out.data_ptr(), mt, nt, W // 8, st))
+    return out

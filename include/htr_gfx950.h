@@ -1,0 +1,100 @@
+/*
+ * C ABI of libhtr_gfx950.so: the MI355X (gfx950) execution path for HTR-W1 packed linears.
+ *
+ * Plain pointers and sizes only.  All pointers except `problems` arrays are DEVICE pointers
+ * on the current HIP device; `stream` is a hipStream_t passed as void* (NULL = default
+ * stream).  Every call is asynchronous on `stream`, allocates nothing and never
+ * synchronises.  Return value: 0 on success, otherwise an htr_status code whose text
+ * htr_strerror() returns.
+ *
+ * Tensors use the HTR-W1 wire layout of the reference (docs/FORMAT.md:25-32):
+ *   qweight int32 [m/16, n/16, 8K]  (uint32 bit patterns), K = 2..8
+ *   scales  float16 [m]
+ *   su      uint8 [n/8],  sv uint8 [m/8]   bit j%8 (LSB first) of byte j/8 set -> sign -1
+ * m and n are multiples of 128.
+ *
+ * Each entry point names the reference interface it stands in for (paths relative to the
+ * reference tree).
+ */
+#ifndef HTR_GFX950_H
+#define HTR_GFX950_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+  HTR_OK = 0,
+  HTR_ERR_NULL = 1,       /* a required pointer is NULL */
+  HTR_ERR_K = 2,          /* K outside 2..8 */
+  HTR_ERR_SHAPE = 3,      /* m or n not a positive multiple of 128 */
+  HTR_ERR_BATCH = 4,      /* M outside 1..HTR_MAX_BATCH */
+  HTR_ERR_DTYPE = 5,      /* dtype code not one of HTR_BF16/HTR_F16/HTR_F32 */
+  HTR_ERR_WORKSPACE = 6,  /* workspace too small or misaligned */
+  HTR_ERR_ALIGN = 7,      /* a tensor pointer is not aligned as required */
+  HTR_ERR_LAUNCH = 8,     /* the HIP runtime refused the launch (see htr_last_hip_error) */
+  HTR_ERR_SPLIT = 9,      /* explicit split count not usable for this shape */
+  HTR_ERR_COUNT = 10      /* grouped call: count outside 1..HTR_MAX_GROUP */
+} htr_status;
+
+/* element type codes; same numbering as the reference's out-dtype map (htr/ops.py:79,94) */
+enum { HTR_BF16 = 0, HTR_F16 = 1, HTR_F32 = 2 };
+
+#define HTR_MAX_BATCH 32   /* activation rows one htr_linear launch accepts */
+#define HTR_MAX_GROUP 4096 /* problems one htr_linear_grouped launch accepts */
+
+const char* htr_strerror(int status);
+/* hipError_t value of the last failed launch on this thread (0 if none) */
+int htr_last_hip_error(void);
+int htr_abi_version(void);
+
+/* CBSCALE = 1/sqrt(mean_s v(s)^2) as the float32 the kernels multiply by.
+ * Reference: wire.cbscale(), htr/wire.py:28-30 (used as ops.CB, htr/ops.py:7). */
+float htr_cbscale(void);
+
+/*
+ * Bytes of zero-initialised device workspace htr_linear needs for this problem (counters +
+ * split partials).  The caller allocates it once, zeroes it once, and may reuse it for any
+ * later call whose requirement is not larger, as long as calls that share a workspace are
+ * ordered on one stream: kernels leave the counter words zero on exit.
+ * Reference: the per-device int32[65536] counter tensor (htr/ops.py:24-28) plus the
+ * `part` tensors the extension allocates per call (htr/csrc/htr_kernels.cu:1145).
+ * nsplit: 0 = library policy, >0 = explicit split count (as in htr_linear).
+ */
+size_t htr_workspace_bytes(int m, int n, int K, int M, int nsplit);
+
+/*
+ * y[M, m] = x[M, n] @ W^T (+ bias) for an HTR-W1 weight, one fused launch: input sign flip +
+ * H128, trellis decode, row scale, fp32-accumulated product, output H128 + sign, bias, cast.
+ * Reference: the decode branch of _linear_impl (htr/ops.py:75-76, :94-98), i.e.
+ * prologue + gemv_epi / gemv_fused (htr/csrc/htr_kernels.cu:972-987, :1134-1173, :1034-1064).
+ *   x      [M, n] row-major, x_dtype (bf16 / f16 / f32)
+ *   bias   [m] in y_dtype, or NULL
+ *   y      [M, m] row-major, y_dtype
+ *   nsplit 0 = library policy; >0 = number of column splits to use
+ */
+int htr_linear(const void* qweight, const void* scales, const void* su, const void* sv,
+               const void* x, const void* bias, void* y,
+               int m, int n, int K, int M, int x_dtype, int y_dtype, int nsplit,
+               void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Integer decode, tile order: out[tile, t] = v(s_t) as int16, tile = ti*(n/16)+tj, t = 16r+c.
+ * Reference: decode_raw (htr/csrc/htr_kernels.cu:943-951, kernel :154-172).
+ */
+int htr_decode_raw(const void* qweight, void* out_i16, int64_t ntiles, int K, void* stream);
+
+/*
+ * Rotated-domain Q[m, n] float32 = cb[s] * float32(scale_row), bit-exact with the
+ * reference's CPU decoder.  Reference: wire.dequant_Q (htr/wire.py:95-102); the GPU
+ * counterpart there is dequant_f16 (htr/csrc/htr_kernels.cu:932-941), which rounds to f16.
+ */
+int htr_dequant_q(const void* qweight, const void* scales, void* out_f32, int mt, int nt, int K, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HTR_GFX950_H */

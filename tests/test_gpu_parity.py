@@ -1,0 +1,186 @@
+"""GPU parity: the gfx950 library (through its C ABI) against the CPU oracle on identical seeded inputs.
+
+Bars: integer decode (int16 v) and float32 Q bit-exact; float32-output linear within 1e-3 of the float64
+decode-then-matmul, measured as max|y - y_ref| / max|y_ref|; bf16 output within one bf16 ulp of bf16(y_ref).
+"""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+REL_TOL = 1e-3
+
+
+@pytest.fixture(scope="module")
+def dev():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from htr_amd import _native
+    _native.lib()          # must load: there is no fallback path
+    return torch.device("cuda:0")
+
+
+def _case(m, n, K, M, seed, dtype=torch.bfloat16):
+    from htr_amd import wire
+    qw, sc, su, sv = wire.synth_linear(m, n, K, seed)
+    x = wire.synth_activation(M, n, seed + 7, dtype)
+    return qw, sc, su, sv, x
+
+
+def _ref(oracle, qw, sc, su, sv, x, bias=None):
+    return oracle.c_linear(x.float().numpy(), qw.numpy(), sc.numpy(), su.numpy(), sv.numpy(),
+                           None if bias is None else bias.float().numpy().astype(np.float64))
+
+
+def _rel(y, ref):
+    return float(np.abs(y - ref).max() / np.abs(ref).max())
+
+
+@pytest.mark.parametrize("K", [2, 3, 4, 5, 6, 7, 8])
+def test_decode_raw_bit_exact(dev, oracle, K):
+    from htr_amd import ops, wire
+    print(f"decode_raw K={K}", flush=True)
+    qw = wire.synth_linear(256, 384, K, 100 + K)[0]
+    got = ops.decode_raw(qw.to(dev)).cpu().numpy()
+    assert np.array_equal(got, oracle.c_decode_raw(qw.numpy()))
+
+
+@pytest.mark.parametrize("K", [2, 3, 4, 5])
+def test_decode_raw_edge_streams(dev, oracle, K):
+    from htr_amd import ops
+    print(f"decode_raw edges K={K}", flush=True)
+    zeros = torch.zeros(3, 5, 8 * K, dtype=torch.int32)
+    ones = torch.full((3, 5, 8 * K), -1, dtype=torch.int32)
+    assert torch.all(ops.decode_raw(zeros.to(dev)) == -303)
+    assert torch.all(ops.decode_raw(ones.to(dev)) == -16)
+    # one set bit anywhere in the stream, including the wrap region at both ends
+    words = torch.zeros(256 * K, 8 * K, dtype=torch.int64)
+    for p in range(256 * K):
+        words[p, p >> 5] = 1 << (31 - (p & 31))
+    words = torch.where(words >= 2 ** 31, words - 2 ** 32, words).to(torch.int32).reshape(256 * K, 1, 8 * K)
+    got = ops.decode_raw(words.to(dev)).cpu().numpy()
+    assert np.array_equal(got, oracle.c_decode_raw(words.numpy()))
+
+
+@pytest.mark.parametrize("K", [2, 3, 4, 5, 8])
+def test_dequant_q_bit_exact(dev, oracle, K):
+    from htr_amd import ops, wire
+    print(f"dequant_q K={K}", flush=True)
+    qw, sc, _, _ = wire.synth_linear(256, 512, K, 200 + K)
+    got = ops.dequant_q(qw.to(dev), sc.to(dev)).cpu().numpy()
+    want = oracle.c_dequant_q(qw.numpy(), sc.numpy())
+    assert got.dtype == np.float32 and np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+@pytest.mark.parametrize("K", [2, 3, 4, 5])
+@pytest.mark.parametrize("M", [1, 2, 3, 4, 8])
+@pytest.mark.parametrize("shape", [(256, 384), (1024, 4096), (4096, 1024)])
+def test_linear_f32_out_within_tolerance(dev, oracle, K, M, shape):
+    from htr_amd import ops
+    m, n = shape
+    print(f"linear f32 K={K} M={M} {m}x{n}", flush=True)
+    qw, sc, su, sv, x = _case(m, n, K, M, 1000 * K + 10 * M + m % 7)
+    y = ops.linear_f32out(x.to(dev), qw.to(dev), sc.to(dev), su.to(dev), sv.to(dev)).cpu().numpy()
+    ref = _ref(oracle, qw, sc, su, sv, x)
+    assert y.shape == ref.shape
+    assert _rel(y, ref) <= REL_TOL, _rel(y, ref)
+
+
+@pytest.mark.parametrize("K,M", [(3, 16), (4, 9), (4, 16), (4, 32), (3, 32), (5, 17), (4, 45)])
+def test_linear_small_batch_blocks(dev, oracle, K, M):
+    from htr_amd import ops
+    print(f"linear batch K={K} M={M}", flush=True)
+    qw, sc, su, sv, x = _case(512, 1024, K, M, 31 * K + M)
+    y = ops.linear_f32out(x.to(dev), qw.to(dev), sc.to(dev), su.to(dev), sv.to(dev)).cpu().numpy()
+    ref = _ref(oracle, qw, sc, su, sv, x)
+    assert _rel(y, ref) <= REL_TOL, _rel(y, ref)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_linear_api_dtypes_bias_and_batch_dims(dev, oracle, dtype):
+    from htr_amd import ops
+    print(f"linear api dtype={dtype}", flush=True)
+    qw, sc, su, sv, x = _case(384, 256, 4, 6, 77, dtype)
+    bias = torch.randn(384, generator=torch.Generator().manual_seed(5)).to(dtype)
+    x3 = x.reshape(2, 3, 256)
+    y = ops.linear(x3.to(dev), qw.to(dev), sc.to(dev), su.to(dev), sv.to(dev), bias.to(dev))
+    assert y.dtype == dtype and tuple(y.shape) == (2, 3, 384)
+    ref = _ref(oracle, qw, sc, su, sv, x, bias)
+    got = y.float().cpu().numpy().reshape(6, 384)
+    if dtype == torch.float32:
+        assert _rel(got, ref) <= REL_TOL
+    else:
+        want = torch.from_numpy(ref).to(dtype)
+        # one ulp of the output type around the rounded reference, plus the fp32-path tolerance
+        ulp = (torch.nextafter(want.float().abs().to(dtype), torch.tensor(float("inf"), dtype=dtype)).float()
+               - want.float().abs())
+        err = (torch.from_numpy(got) - want.float()).abs()
+        slack = REL_TOL * float(np.abs(ref).max())
+        assert bool(torch.all(err <= ulp + slack))
+
+
+def test_bf16_output_within_one_ulp(dev, oracle):
+    from htr_amd import ops
+    print("linear bf16 ulp", flush=True)
+    qw, sc, su, sv, x = _case(1024, 2048, 4, 1, 4242)
+    d = [t.to(dev) for t in (qw, sc, su, sv)]
+    y = ops.linear(x.to(dev), *d).float().cpu()
+    y32 = ops.linear_f32out(x.to(dev), *d).cpu()
+    assert torch.equal(y, y32.bfloat16().float())            # the cast is round-to-nearest-even of the f32 result
+    ref = torch.from_numpy(_ref(oracle, qw, sc, su, sv, x))
+    want = ref.bfloat16().float()
+    ulp = want.abs() * 2.0 ** -7 + 1e-30
+    assert bool(torch.all((y - want).abs() <= ulp))
+
+
+def test_large_activations_do_not_overflow(dev, oracle):
+    from htr_amd import ops
+    print("linear large activations", flush=True)
+    qw, sc, su, sv, x = _case(256, 512, 4, 2, 99, torch.float32)
+    x = x * 1e4
+    x[1] *= 1e-9                                            # one huge row, one tiny row
+    y = ops.linear_f32out(x.to(dev), qw.to(dev), sc.to(dev), su.to(dev), sv.to(dev)).cpu().numpy()
+    ref = _ref(oracle, qw, sc, su, sv, x)
+    assert np.all(np.isfinite(y))
+    for r in range(2):
+        assert _rel(y[r], ref[r]) <= REL_TOL
+
+
+def test_zero_rows_and_repeatability(dev):
+    from htr_amd import ops
+    print("linear M=0 / repeat", flush=True)
+    qw, sc, su, sv, x = _case(512, 512, 4, 4, 5)
+    d = [t.to(dev) for t in (qw, sc, su, sv)]
+    assert tuple(ops.linear(x[:0].to(dev), *d).shape) == (0, 512)
+    xs = x.to(dev)
+    a = ops.linear_f32out(xs, *d)
+    for _ in range(5):                                     # counters reset themselves; result is deterministic
+        assert torch.equal(a, ops.linear_f32out(xs, *d))
+
+
+def test_errors(dev):
+    from htr_amd import ops
+    qw, sc, su, sv, x = _case(256, 256, 4, 1, 6)
+    d = [t.to(dev) for t in (qw, sc, su, sv)]
+    with pytest.raises(RuntimeError):
+        ops.linear(x.to(dev)[:, :128].contiguous(), *d)
+    with pytest.raises(RuntimeError):
+        ops.linear(x.to(dev), d[0], d[1].float(), d[2], d[3])
+    with pytest.raises(RuntimeError):
+        ops.linear(x.to(dev), d[0][:, :, :8].contiguous(), d[1], d[2], d[3])      # K = 1
+
+
+@pytest.mark.parametrize("K,m,n", [(4, 4096, 4096), (2, 4096, 4096), (5, 4096, 4096), (4, 14336, 4096),
+                                   (4, 4096, 14336), (3, 14336, 4096)])
+def test_full_size_shapes(dev, oracle, K, m, n):
+    from htr_amd import ops
+    print(f"full size K={K} {m}x{n}", flush=True)
+    qw, sc, su, sv, x = _case(m, n, K, 1, 20261125 + K)
+    d = [t.to(dev) for t in (qw, sc, su, sv)]
+    y = ops.linear_f32out(x.to(dev), *d).cpu().numpy()
+    ref = _ref(oracle, qw, sc, su, sv, x)
+    assert _rel(y, ref) <= REL_TOL, _rel(y, ref)
+    # linearity in x, a size-independent property: f(2x) == 2 f(x) exactly (power-of-two scaling)
+    y2 = ops.linear_f32out((x * 2).to(dev), *d).cpu().numpy()
+    assert np.array_equal(y2, 2 * y)

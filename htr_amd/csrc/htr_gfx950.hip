@@ -146,17 +146,19 @@ struct LinearArgs {
   const void* x;
   const void* bias;
   void* y;
-  float* part;
-  uint32_t* cnt;
+  float* part;      // [m/128][ns][M][128] split partials
+  uint32_t* cnt;    // [m/128] arrival counters, zero on entry and on exit
   int m, n, M, ns, bps, x_dtype, y_dtype;
   float cbscale;
 };
 
-// LDS layout (dynamic): [xt: (M + 1) rows x row_halves f16][amax: 32 u32][sc: 32 f32][xs: M * bps f32][yt: M * 128 f32]
+// LDS layout (dynamic): [xt: (M + 1) rows x row_halves f16][pmax: M * bps f32][xs: M * bps f32]
 __host__ __device__ inline int xt_row_halves(int bps) { return bps * 128 + 8; }   // +8 halves: rows land on different banks
 __host__ __device__ inline size_t lds_bytes(int M, int bps) {
-  return (size_t)(M + 1) * xt_row_halves(bps) * 2 + 32 * 4 + 32 * 4 + (size_t)M * bps * 4 + (size_t)M * 128 * 4;
+  return (size_t)(M + 1) * xt_row_halves(bps) * 2 + (size_t)M * bps * 4 * 2;
 }
+
+constexpr int PAIR_REGS = 4;   // (activation row, 128-column block) pairs a wave keeps in registers across the barrier
 
 template <int K, int MB, int P>
 __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
@@ -169,10 +171,8 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
   const int rowh = xt_row_halves(a.bps);
 
   _Float16* xt = (_Float16*)lds;
-  uint32_t* s_amax = (uint32_t*)(lds + (size_t)(M + 1) * rowh * 2);
-  float* s_sc = (float*)(s_amax + 32);
-  float* s_xs = s_sc + 32;
-  float* s_y = s_xs + M * a.bps;
+  float* s_pmax = (float*)(lds + (size_t)(M + 1) * rowh * 2);
+  float* s_xs = s_pmax + M * a.bps;
 
   // ---- start the weight stream first: everything below overlaps with these loads
   const uint32_t* wp = a.qw + ((size_t)(rb * 8 + w) * nt + (size_t)8 * b0) * (8 * K) + lane * K;
@@ -182,32 +182,55 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
   for (int p = 0; p < P; ++p)
     if (p < nb) load_stream<K>(wp + (size_t)p * STEP_DWORDS, buf[p]);
 
-  // ---- input rotation of this split's columns: x~ = f16( H128(su . x) / sqrt(128) / sc ), sc a power of two per row
-  if (threadIdx.x < 32) s_amax[threadIdx.x] = 0u;
-  for (int i = threadIdx.x; i < rowh / 2; i += WG_THREADS) ((uint32_t*)(xt + (size_t)M * rowh))[i] = 0u;   // zero row
-  __syncthreads();
+  // ---- input rotation of this split's columns: x~ = f16( H128(su . x) / sqrt(128) / sc ), sc a power of two per row.
+  // Pass 1 loads x (sign applied) and publishes max|x| per (row, block); pass 2 rotates, scales, converts.
   const int npairs = M * nb;
-  for (int pi = w; pi < npairs; pi += WG_WAVES) {
+  float xa[PAIR_REGS], xb[PAIR_REGS];
+  for (int i = threadIdx.x; i < rowh / 2; i += WG_THREADS) ((uint32_t*)(xt + (size_t)M * rowh))[i] = 0u;   // zero row
+#pragma unroll
+  for (int t = 0; t < PAIR_REGS; ++t) {
+    const int pi = w + t * WG_WAVES;
+    if (pi < npairs) {
+      const int mrow = pi / nb, bl = pi - mrow * nb, col = (b0 + bl) * 128;
+      const size_t base = (size_t)mrow * a.n + col;
+      xa[t] = load_elem(a.x, a.x_dtype, base + lane) * sign_of(a.su, col + lane);
+      xb[t] = load_elem(a.x, a.x_dtype, base + lane + 64) * sign_of(a.su, col + lane + 64);
+      float mx = fmaxf(fabsf(xa[t]), fabsf(xb[t]));
+#pragma unroll
+      for (int h = 32; h >= 1; h >>= 1) mx = fmaxf(mx, lane_xor(mx, h));
+      if (lane == 0) s_pmax[pi] = mx;
+    }
+  }
+  for (int pi = w + PAIR_REGS * WG_WAVES; pi < npairs; pi += WG_WAVES) {   // more pairs than registers: max only, reload later
     const int mrow = pi / nb, bl = pi - mrow * nb;
     const size_t base = (size_t)mrow * a.n + (size_t)(b0 + bl) * 128;
     float mx = fmaxf(fabsf(load_elem(a.x, a.x_dtype, base + lane)), fabsf(load_elem(a.x, a.x_dtype, base + lane + 64)));
 #pragma unroll
     for (int h = 32; h >= 1; h >>= 1) mx = fmaxf(mx, lane_xor(mx, h));
-    if (lane == 0) atomicMax(&s_amax[mrow], __float_as_uint(mx));
+    if (lane == 0) s_pmax[pi] = mx;
   }
   __syncthreads();
-  for (int pi = w; pi < npairs; pi += WG_WAVES) {
-    const int mrow = pi / nb, bl = pi - mrow * nb;
-    const int col = (b0 + bl) * 128;
-    const size_t base = (size_t)mrow * a.n + col;
-    // |H128 x| / sqrt(128) <= sqrt(128) * amax; keep that bound in (8192, 16384] so f16 neither overflows nor
+  for (int t = 0, pi = w; pi < npairs; ++t, pi += WG_WAVES) {
+    const int mrow = pi / nb, bl = pi - mrow * nb, col = (b0 + bl) * 128;
+    float amax = 0.f;
+    for (int k = 0; k < nb; ++k) amax = fmaxf(amax, s_pmax[mrow * nb + k]);
+    // |H128 x| / sqrt(128) <= sqrt(128) * max|x|; keep that bound in (8192, 16384] so f16 neither overflows nor
     // loses small activations to denormals
-    const float bound = __uint_as_float(s_amax[mrow]) * SQRT128;
+    const float bound = amax * SQRT128;
     int e = 0;
     if (bound > 0.f && bound < 3.0e38f) e = ilogbf(bound) - 13;
     const float inv_sc = ldexpf(1.f, -e);
-    float va = load_elem(a.x, a.x_dtype, base + lane) * sign_of(a.su, col + lane) * inv_sc;
-    float vb = load_elem(a.x, a.x_dtype, base + lane + 64) * sign_of(a.su, col + lane + 64) * inv_sc;
+    float va, vb;
+    if (t < PAIR_REGS) {
+      va = 0.f; vb = 0.f;
+#pragma unroll
+      for (int u = 0; u < PAIR_REGS; ++u) if (u == t) { va = xa[u]; vb = xb[u]; }
+    } else {
+      const size_t base = (size_t)mrow * a.n + col;
+      va = load_elem(a.x, a.x_dtype, base + lane) * sign_of(a.su, col + lane);
+      vb = load_elem(a.x, a.x_dtype, base + lane + 64) * sign_of(a.su, col + lane + 64);
+    }
+    va *= inv_sc; vb *= inv_sc;
     fwht128_wave(va, vb, lane);
     const _Float16 ha = (_Float16)(va * INV_SQRT128), hb = (_Float16)(vb * INV_SQRT128);
     xt[(size_t)mrow * rowh + bl * 128 + lane] = ha;
@@ -215,10 +238,7 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
     float s = (float)ha + (float)hb;
 #pragma unroll
     for (int h = 32; h >= 1; h >>= 1) s += lane_xor(s, h);
-    if (lane == 0) {
-      s_xs[pi] = s;
-      if (bl == 0) s_sc[mrow] = ldexpf(1.f, e);
-    }
+    if (lane == 0) s_xs[pi] = s;
   }
   __syncthreads();
 
@@ -267,64 +287,71 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
     }
   }
 
-  // ---- fold the two tile parities, remove the 1534 offset, undo the activation scale -> this split's partial
+  // ---- fold the two tile parities, remove the 1534 offset, undo the activation scale -> this wave's strip partial.
   // D[i][c] sits in lane c + 16 * (i / 4), register i % 4.  Row pair q is D row q (even tiles, column 2r) plus
-  // D row q + 8 (odd tiles, column 2r + 1): lane (g', c) with g' < 2 and c even adds lane + 33.
+  // D row q + 8 (odd tiles, column 2r + 1): lane (g', c) with g' < 2 and c even adds lane + 33 and then holds rows
+  // 8g' .. 8g' + 7 of the strip for activation row c / 2.
+  // Partials and the arrival counter use agent-scope (write-through / L2-bypassing) accesses, so no cache-wide
+  // writeback or invalidate is needed.
+  float* mypart = a.part + ((size_t)(rb * a.ns + sp) * M) * 128;
   {
     const int partner = ((lane + 33) & 63) << 2;
     const bool keeper = g < 2 && (n16 & 1) == 0;
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
       const int mrow = mb * 8 + (n16 >> 1);
+      const bool live = keeper && mrow < M;
       float xs = 0.f, sc = 0.f;
-      if (keeper && mrow < M) {
-        for (int bl = 0; bl < nb; ++bl) xs += s_xs[mrow * nb + bl];
-        sc = s_sc[mrow];
+      if (live) {
+        float amax = 0.f;
+        for (int bl = 0; bl < nb; ++bl) { xs += s_xs[mrow * nb + bl]; amax = fmaxf(amax, s_pmax[mrow * nb + bl]); }
+        const float bound = amax * SQRT128;
+        int e = 0;
+        if (bound > 0.f && bound < 3.0e38f) e = ilogbf(bound) - 13;
+        sc = ldexpf(1.f, e);
       }
+      float out[8];
 #pragma unroll
       for (int rr = 0; rr < 2; ++rr)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
           const float mine = acc[mb][rr][j];
           const float other = __uint_as_float((uint32_t)__builtin_amdgcn_ds_bpermute(partner, (int)__float_as_uint(mine)));
-          if (keeper && mrow < M) s_y[mrow * 128 + 16 * w + 2 * (4 * g + j) + rr] = ((mine + other) - 1534.f * xs) * sc;
+          out[2 * j + rr] = ((mine + other) - 1534.f * xs) * sc;
         }
-    }
-  }
-  __syncthreads();
-
-  if (a.ns > 1) {
-    float* mypart = a.part + ((size_t)(rb * a.ns + sp) * M) * 128;
-    for (int i = threadIdx.x; i < M * 128; i += WG_THREADS) mypart[i] = s_y[i];
-    __threadfence();
-    __syncthreads();
-    __shared__ int s_last;
-    if (threadIdx.x == 0) s_last = (atomicAdd(&a.cnt[rb], 1u) == (uint32_t)(a.ns - 1));
-    __syncthreads();
-    if (!s_last) return;
-    __threadfence();
-  }
-
-  // ---- output side: sum the splits in a fixed order, row scale, H128, sv, bias, cast
-  for (int mrow = w; mrow < M; mrow += WG_WAVES) {
-    float v0, v1;
-    if (a.ns > 1) {
-      v0 = 0.f; v1 = 0.f;
-      const float* pp = a.part + ((size_t)rb * a.ns * M + mrow) * 128;
-      for (int s = 0; s < a.ns; ++s) {
-        v0 += __builtin_nontemporal_load(pp + (size_t)s * M * 128 + lane);
-        v1 += __builtin_nontemporal_load(pp + (size_t)s * M * 128 + lane + 64);
+      if (live) {
+        float* dst = mypart + mrow * 128 + 16 * w + 8 * g;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) __hip_atomic_store(dst + i, out[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
-    } else {
-      v0 = s_y[mrow * 128 + lane];
-      v1 = s_y[mrow * 128 + lane + 64];
     }
-    const int r0 = rb * 128 + lane, r1 = r0 + 64;
-    v0 *= f16_bits_to_float(a.scales[r0]) * a.cbscale;
-    v1 *= f16_bits_to_float(a.scales[r1]) * a.cbscale;
+  }
+  // device-scope stores are acknowledged once written through; wait for every acknowledgement before the barrier
+  // lets thread 0 announce the workgroup (a cache-wide writeback would also do, at many times the cost).
+  // One arrival per workgroup: atomics on one address serialise, so the count is kept as low as possible.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __shared__ uint32_t s_old;
+  __syncthreads();
+  if (threadIdx.x == 0) s_old = __hip_atomic_fetch_add(&a.cnt[rb], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __syncthreads();
+  if (s_old != (uint32_t)(a.ns - 1)) return;
+
+  // ---- last workgroup of the row block: sum the splits in a fixed order, row scale, H128, sv, bias, cast
+  if (threadIdx.x == 0) __hip_atomic_store(&a.cnt[rb], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next call
+  const int r0 = rb * 128 + lane, r1 = r0 + 64;
+  const float rs0 = f16_bits_to_float(a.scales[r0]) * a.cbscale, rs1 = f16_bits_to_float(a.scales[r1]) * a.cbscale;
+  const float sg0 = sign_of(a.sv, r0), sg1 = sign_of(a.sv, r1);
+  for (int mrow = w; mrow < M; mrow += WG_WAVES) {
+    float v0 = 0.f, v1 = 0.f;
+    const float* pp = a.part + ((size_t)rb * a.ns * M + mrow) * 128;
+    for (int s = 0; s < a.ns; ++s) {
+      v0 += __hip_atomic_load(pp + (size_t)s * M * 128 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      v1 += __hip_atomic_load(pp + (size_t)s * M * 128 + lane + 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    v0 *= rs0; v1 *= rs1;
     fwht128_wave(v0, v1, lane);
-    v0 = v0 * INV_SQRT128 * sign_of(a.sv, r0);
-    v1 = v1 * INV_SQRT128 * sign_of(a.sv, r1);
+    v0 = v0 * INV_SQRT128 * sg0;
+    v1 = v1 * INV_SQRT128 * sg1;
     if (a.bias != nullptr) {
       v0 += load_elem(a.bias, a.y_dtype, r0);
       v1 += load_elem(a.bias, a.y_dtype, r1);
@@ -332,7 +359,6 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
     store_elem(a.y, a.y_dtype, (size_t)mrow * a.m + r0, v0);
     store_elem(a.y, a.y_dtype, (size_t)mrow * a.m + r1, v1);
   }
-  if (a.ns > 1 && threadIdx.x == 0) a.cnt[rb] = 0u;   // leave the counter ready for the next call
 }
 
 // ------------------------------------------------------------------------------------------------ debug decodes
@@ -428,7 +454,10 @@ inline bool make_plan(int m, int n, int M, int nsplit, Plan& pl) {
   return true;
 }
 
-inline size_t counters_bytes(int m) { return (((size_t)(m / 128) * 4) + 255) / 256 * 256; }
+// fixed-size counter region at the start of the workspace, so that partials of one call can never land on words a
+// later call with a different shape uses as counters
+constexpr int MAX_ROW_BLOCKS = 16384;
+inline size_t counters_bytes() { return (size_t)MAX_ROW_BLOCKS * 4; }
 
 template <int K, int MB> int launch_linear_kmb(const LinearArgs& a, int grid, size_t lds, hipStream_t st) {
   constexpr int P = K <= 4 ? 4 : (K <= 6 ? 3 : 2);
@@ -491,11 +520,11 @@ int htr_abi_version(void) { return 1; }
 float htr_cbscale(void) { return (float)(1.0 / __builtin_sqrt(MEAN_SQ)); }
 
 size_t htr_workspace_bytes(int m, int n, int K, int M, int nsplit) {
-  if (K < 2 || K > 8 || m <= 0 || n <= 0 || m % 128 || n % 128 || M < 1 || M > HTR_MAX_BATCH) return 0;
+  if (K < 2 || K > 8 || m <= 0 || n <= 0 || m % 128 || n % 128 || m / 128 > MAX_ROW_BLOCKS || M < 1 || M > HTR_MAX_BATCH) return 0;
   Plan pl;
   if (!make_plan(m, n, M, nsplit, pl)) return 0;
-  size_t bytes = counters_bytes(m);
-  if (pl.ns > 1) bytes += (size_t)(m / 128) * pl.ns * M * 128 * sizeof(float);
+  size_t bytes = counters_bytes();
+  bytes += (size_t)(m / 128) * pl.ns * M * 128 * sizeof(float);
   return bytes;
 }
 
@@ -504,7 +533,7 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
                size_t workspace_bytes, void* stream) {
   if (!qweight || !scales || !su || !sv || !x || !y) return HTR_ERR_NULL;
   if (K < 2 || K > 8) return HTR_ERR_K;
-  if (m <= 0 || n <= 0 || m % 128 || n % 128) return HTR_ERR_SHAPE;
+  if (m <= 0 || n <= 0 || m % 128 || n % 128 || m / 128 > MAX_ROW_BLOCKS) return HTR_ERR_SHAPE;
   if (M < 1 || M > HTR_MAX_BATCH) return HTR_ERR_BATCH;
   if (!dtype_ok(x_dtype) || !dtype_ok(y_dtype)) return HTR_ERR_DTYPE;
   if (((uintptr_t)qweight & 15) || ((uintptr_t)scales & 1) || ((uintptr_t)x & (x_dtype == HTR_F32 ? 3 : 1)) ||
@@ -519,7 +548,7 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
   a.qw = (const uint32_t*)qweight; a.scales = (const uint16_t*)scales; a.su = (const uint8_t*)su; a.sv = (const uint8_t*)sv;
   a.x = x; a.bias = bias; a.y = y;
   a.cnt = (uint32_t*)workspace;
-  a.part = (float*)((unsigned char*)workspace + counters_bytes(m));
+  a.part = (float*)((unsigned char*)workspace + counters_bytes());
   a.m = m; a.n = n; a.M = M; a.ns = pl.ns; a.bps = pl.bps; a.x_dtype = x_dtype; a.y_dtype = y_dtype;
   a.cbscale = htr_cbscale();
   const int grid = (m / 128) * pl.ns;

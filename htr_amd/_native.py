@@ -23,6 +23,7 @@ SIGNATURES = {
     "htr_abi_version": (_i, []),
     "htr_cbscale": (ctypes.c_float, []),
     "htr_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
+    "htr_linear_plan": (_i, [_i, _i, _i, _i, _i, ctypes.POINTER(ctypes.c_int)]),
     "htr_linear": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
     "htr_decode_raw": (_i, [_vp, _vp, _i64, _i, _vp]),
     "htr_dequant_q": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),

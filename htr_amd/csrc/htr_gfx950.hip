@@ -64,18 +64,58 @@ __device__ __forceinline__ void store_elem(void* p, int dtype, size_t idx, float
   else ((float*)p)[idx] = v;
 }
 __device__ __forceinline__ float sign_of(const uint8_t* bits, int j) { return ((bits[j >> 3] >> (j & 7)) & 1) ? -1.f : 1.f; }
-__device__ __forceinline__ float lane_xor(float v, int mask) { return __shfl_xor(v, mask, 64); }
+// ---- cross-lane exchange without LDS round trips: DPP for lane xor 1, 2, 4, 8; gfx950 row swaps for 16 and 32
+template <int CTRL> __device__ __forceinline__ float dpp_mov(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, false));
+}
+template <int H> __device__ __forceinline__ float lane_xor_dpp(float v) {
+  if constexpr (H == 1) return dpp_mov<0xB1>(v);                   // quad_perm [1,0,3,2]
+  else if constexpr (H == 2) return dpp_mov<0x4E>(v);              // quad_perm [2,3,0,1]
+  else if constexpr (H == 4) return dpp_mov<0x141>(dpp_mov<0x1B>(v));   // quad reverse (xor 3) then row_half_mirror (xor 7)
+  else return dpp_mov<0x128>(v);                                   // row_ror:8 == xor 8 inside a row of 16
+}
+// values of the two 16-lane (or 32-lane) halves that lane and lane ^ 16 (^ 32) belong to: first = even half's value,
+// second = odd half's value, both seen from every lane of the pair
+typedef uint32_t u2s __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void halves16(float v, float& even, float& odd) {
+  const uint32_t u = __float_as_uint(v);
+  const u2s r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  even = __uint_as_float(r.x); odd = __uint_as_float(r.y);
+}
+__device__ __forceinline__ void halves32(float v, float& even, float& odd) {
+  const uint32_t u = __float_as_uint(v);
+  const u2s r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  even = __uint_as_float(r.x); odd = __uint_as_float(r.y);
+}
+template <int H> __device__ __forceinline__ void butterfly_dpp(float& a, int lane) {
+  const float p = lane_xor_dpp<H>(a);
+  a = (lane & H) ? (p - a) : (a + p);
+}
+__device__ __forceinline__ void butterfly16(float& a, int lane) { float e, o; halves16(a, e, o); a = (lane & 16) ? (e - o) : (e + o); }
+__device__ __forceinline__ void butterfly32(float& a, int lane) { float e, o; halves32(a, e, o); a = (lane & 32) ? (e - o) : (e + o); }
 
 // 128-point Walsh-Hadamard butterfly network over one wave: lane holds elements `lane` (a) and `lane + 64` (b).
 __device__ __forceinline__ void fwht128_wave(float& a, float& b, int lane) {
   float t = a + b; b = a - b; a = t;
-#pragma unroll
-  for (int h = 32; h >= 1; h >>= 1) {
-    const float pa = lane_xor(a, h), pb = lane_xor(b, h);
-    const bool up = (lane & h) != 0;
-    a = up ? (pa - a) : (a + pa);
-    b = up ? (pb - b) : (b + pb);
-  }
+  butterfly_dpp<1>(a, lane); butterfly_dpp<1>(b, lane);
+  butterfly_dpp<2>(a, lane); butterfly_dpp<2>(b, lane);
+  butterfly_dpp<4>(a, lane); butterfly_dpp<4>(b, lane);
+  butterfly_dpp<8>(a, lane); butterfly_dpp<8>(b, lane);
+  butterfly16(a, lane); butterfly16(b, lane);
+  butterfly32(a, lane); butterfly32(b, lane);
+}
+// all-lanes reductions over the wave, fixed order
+__device__ __forceinline__ float wave_sum(float v) {
+  v += lane_xor_dpp<1>(v); v += lane_xor_dpp<2>(v); v += lane_xor_dpp<4>(v); v += lane_xor_dpp<8>(v);
+  float e, o;
+  halves16(v, e, o); v = e + o;
+  halves32(v, e, o); return e + o;
+}
+__device__ __forceinline__ float wave_max(float v) {
+  v = fmaxf(v, lane_xor_dpp<1>(v)); v = fmaxf(v, lane_xor_dpp<2>(v)); v = fmaxf(v, lane_xor_dpp<4>(v)); v = fmaxf(v, lane_xor_dpp<8>(v));
+  float e, o;
+  halves16(v, e, o); v = fmaxf(e, o);
+  halves32(v, e, o); return fmaxf(e, o);
 }
 
 // ------------------------------------------------------------------------------------------------ stream loads
@@ -146,27 +186,44 @@ struct LinearArgs {
   const void* x;
   const void* bias;
   void* y;
-  float* part;      // [m/128][ns][M][128] split partials
-  uint32_t* cnt;    // [m/128] arrival counters, zero on entry and on exit
-  int m, n, M, ns, bps, x_dtype, y_dtype;
+  uint32_t* cnt;    // [m/128] arrival counters (election by counter only); zero on entry and on exit
+  float* part;      // [m/128][ns][2][M][128] split partials per tile parity; all-zero on entry and on exit
+  int m, n, M;
+  int ns;           // column splits
+  int bps;          // 128-column blocks per split
+  int rpw;          // row blocks per workgroup
+  int by_counter;   // 1: elect the finisher of a row block with an arrival counter; 0: by reading every split's slots
+  int x_dtype, y_dtype;
   float cbscale;
 };
 
-// LDS layout (dynamic): [xt: (M + 1) rows x row_halves f16][pmax: M * bps f32][xs: M * bps f32]
+constexpr int MAX_RPW = 32;    // row blocks one workgroup may walk
+constexpr int PAIR_REGS = 4;   // (activation row, 128-column block) pairs a wave keeps in registers across the barrier
+
+// LDS layout (dynamic): [xt: (M + 1) rows x row_halves f16][pmax: M * bps f32][xs: M * bps * 2 f32 (per tile parity)]
 __host__ __device__ inline int xt_row_halves(int bps) { return bps * 128 + 8; }   // +8 halves: rows land on different banks
 __host__ __device__ inline size_t lds_bytes(int M, int bps) {
-  return (size_t)(M + 1) * xt_row_halves(bps) * 2 + (size_t)M * bps * 4 * 2;
+  return (size_t)(M + 1) * xt_row_halves(bps) * 2 + (size_t)M * bps * 4 * 3;
 }
 
-constexpr int PAIR_REGS = 4;   // (activation row, 128-column block) pairs a wave keeps in registers across the barrier
+// power-of-two activation scale 2^e with sqrt(128) * amax / 2^e in (8192, 16384]: |H128 x| / sqrt(128) <= sqrt(128) * max|x|,
+// so the rotated activations neither overflow f16 nor fall into its denormals
+__device__ __forceinline__ int scale_exponent(float amax) {
+  const int ex = (int)((__float_as_uint(amax * SQRT128) >> 23) & 0xFFu);
+  if (ex == 0 || ex == 255) return 0;
+  return max(-100, ex - 127 - 13);
+}
+__device__ __forceinline__ float pow2f(int e) { return __uint_as_float((uint32_t)(127 + e) << 23); }
 
 template <int K, int MB, int P>
 __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
   extern __shared__ __align__(16) unsigned char lds[];
+  __shared__ int s_finish[MAX_RPW];
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  const int rb = blockIdx.x / a.ns, sp = blockIdx.x - rb * a.ns;
-  const int nblk = a.n >> 7, nt = a.n >> 4;
+  const int grp = blockIdx.x / a.ns, sp = blockIdx.x - grp * a.ns;
+  const int nblk = a.n >> 7, nt = a.n >> 4, rbs = a.m >> 7;
   const int b0 = sp * a.bps, nb = min(nblk, b0 + a.bps) - b0;
+  const int rb0 = grp * a.rpw, nrb = min(rbs, rb0 + a.rpw) - rb0;
   const int M = a.M;
   const int rowh = xt_row_halves(a.bps);
 
@@ -174,39 +231,51 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
   float* s_pmax = (float*)(lds + (size_t)(M + 1) * rowh * 2);
   float* s_xs = s_pmax + M * a.bps;
 
-  // ---- start the weight stream first: everything below overlaps with these loads
-  const uint32_t* wp = a.qw + ((size_t)(rb * 8 + w) * nt + (size_t)8 * b0) * (8 * K) + lane * K;
-  constexpr int STEP_DWORDS = 64 * K;
-  StreamRegs<K> buf[P];
-#pragma unroll
-  for (int p = 0; p < P; ++p)
-    if (p < nb) load_stream<K>(wp + (size_t)p * STEP_DWORDS, buf[p]);
-
   // ---- input rotation of this split's columns: x~ = f16( H128(su . x) / sqrt(128) / sc ), sc a power of two per row.
   // Pass 1 loads x (sign applied) and publishes max|x| per (row, block); pass 2 rotates, scales, converts.
   const int npairs = M * nb;
   float xa[PAIR_REGS], xb[PAIR_REGS];
   for (int i = threadIdx.x; i < rowh / 2; i += WG_THREADS) ((uint32_t*)(xt + (size_t)M * rowh))[i] = 0u;   // zero row
 #pragma unroll
-  for (int t = 0; t < PAIR_REGS; ++t) {
+  for (int t = 0; t < PAIR_REGS; ++t) {     // x first: loads return in order, and x heads the longest dependency chain
     const int pi = w + t * WG_WAVES;
+    xa[t] = 0.f; xb[t] = 0.f;
     if (pi < npairs) {
       const int mrow = pi / nb, bl = pi - mrow * nb, col = (b0 + bl) * 128;
       const size_t base = (size_t)mrow * a.n + col;
       xa[t] = load_elem(a.x, a.x_dtype, base + lane) * sign_of(a.su, col + lane);
       xb[t] = load_elem(a.x, a.x_dtype, base + lane + 64) * sign_of(a.su, col + lane + 64);
-      float mx = fmaxf(fabsf(xa[t]), fabsf(xb[t]));
+    }
+  }
+
+  // ---- start the weight stream.  The workgroup walks row blocks rb0 .. rb0 + nrb - 1, nb steps each; "virtual
+  // step" v = r * nb + s.  This wave's strip of row block rb0 + r starts at tile row (rb0 + r) * 8 + w.
+  constexpr int STEP_DWORDS = 64 * K;
+  const size_t strip_dwords = (size_t)nt * (8 * K);
+  const uint32_t* wbase = a.qw + ((size_t)(rb0 * 8 + w) * nt + (size_t)8 * b0) * (8 * K) + lane * K;
+  const int total = nrb * nb;
+  StreamRegs<K> buf[P];
+  int pf_r = 0, pf_s = 0;                        // prefetch position
+  auto prefetch = [&](StreamRegs<K>& dst) {
+    load_stream<K>(wbase + (size_t)pf_r * 8 * strip_dwords + (size_t)pf_s * STEP_DWORDS, dst);
+    if (++pf_s == nb) { pf_s = 0; ++pf_r; }
+  };
 #pragma unroll
-      for (int h = 32; h >= 1; h >>= 1) mx = fmaxf(mx, lane_xor(mx, h));
+  for (int p = 0; p < P; ++p)
+    if (p < total) prefetch(buf[p]);
+
+#pragma unroll
+  for (int t = 0; t < PAIR_REGS; ++t) {
+    const int pi = w + t * WG_WAVES;
+    if (pi < npairs) {
+      const float mx = wave_max(fmaxf(fabsf(xa[t]), fabsf(xb[t])));
       if (lane == 0) s_pmax[pi] = mx;
     }
   }
   for (int pi = w + PAIR_REGS * WG_WAVES; pi < npairs; pi += WG_WAVES) {   // more pairs than registers: max only, reload later
     const int mrow = pi / nb, bl = pi - mrow * nb;
     const size_t base = (size_t)mrow * a.n + (size_t)(b0 + bl) * 128;
-    float mx = fmaxf(fabsf(load_elem(a.x, a.x_dtype, base + lane)), fabsf(load_elem(a.x, a.x_dtype, base + lane + 64)));
-#pragma unroll
-    for (int h = 32; h >= 1; h >>= 1) mx = fmaxf(mx, lane_xor(mx, h));
+    const float mx = wave_max(fmaxf(fabsf(load_elem(a.x, a.x_dtype, base + lane)), fabsf(load_elem(a.x, a.x_dtype, base + lane + 64))));
     if (lane == 0) s_pmax[pi] = mx;
   }
   __syncthreads();
@@ -214,12 +283,7 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
     const int mrow = pi / nb, bl = pi - mrow * nb, col = (b0 + bl) * 128;
     float amax = 0.f;
     for (int k = 0; k < nb; ++k) amax = fmaxf(amax, s_pmax[mrow * nb + k]);
-    // |H128 x| / sqrt(128) <= sqrt(128) * max|x|; keep that bound in (8192, 16384] so f16 neither overflows nor
-    // loses small activations to denormals
-    const float bound = amax * SQRT128;
-    int e = 0;
-    if (bound > 0.f && bound < 3.0e38f) e = ilogbf(bound) - 13;
-    const float inv_sc = ldexpf(1.f, -e);
+    const float inv_sc = pow2f(-scale_exponent(amax));
     float va, vb;
     if (t < PAIR_REGS) {
       va = 0.f; vb = 0.f;
@@ -235,39 +299,60 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
     const _Float16 ha = (_Float16)(va * INV_SQRT128), hb = (_Float16)(vb * INV_SQRT128);
     xt[(size_t)mrow * rowh + bl * 128 + lane] = ha;
     xt[(size_t)mrow * rowh + bl * 128 + lane + 64] = hb;
-    float s = (float)ha + (float)hb;
-#pragma unroll
-    for (int h = 32; h >= 1; h >>= 1) s += lane_xor(s, h);
-    if (lane == 0) s_xs[pi] = s;
+    // sum of the rounded x~ per tile parity (element j sits in tile j / 16; lane and lane + 64 share the parity)
+    const float hs = (float)ha + (float)hb;
+    const bool odd_tile = (lane & 16) != 0;
+    const float se = wave_sum(odd_tile ? 0.f : hs), so = wave_sum(odd_tile ? hs : 0.f);
+    if (lane == 0) { s_xs[2 * pi] = se; s_xs[2 * pi + 1] = so; }
   }
   __syncthreads();
 
-  // ---- main loop: one 128-column block (8 tiles of this wave's strip) per step
+  // ---- per-lane constants of the product and of the partial store
+  // MFMA operands: row i = lane % 16 = (tile parity h = i / 8, row pair q = i % 8); B column c = lane % 16 carries
+  // activation row c / 2 and tile parity c % 2; the 16-lane group g = lane / 16 supplies k-slots of tile 2g + parity.
+  // D[i][c] sits in lane c + 16 * (i / 4), register i % 4.  MFMA rows 0..7 (even tiles) are valid in the even
+  // columns c = 2r, rows 8..15 (odd tiles) in the odd columns c = 2r + 1; a valid lane (g', c) holds strip rows
+  // 8 (g' & 1) .. + 7 of activation row c / 2 for parity g' / 2.
   const int g = lane >> 4, n16 = lane & 15;
-  int boff[MB];   // LDS half-index of this lane's B operand for the first block of the split
+  const int par = g >> 1;
+  const bool mine = (n16 & 1) == par;
+  int boff[MB];            // LDS half-index of this lane's B operand for the first block of the split
+  float offs[MB], sc[MB];  // 1534 * sum(x~) of this lane's (row, parity), and the row's activation scale
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
     const int mrow = mb * 8 + (n16 >> 1);
     boff[mb] = (mrow < M ? mrow : M) * rowh + 16 * (2 * g + (n16 & 1));
+    offs[mb] = 0.f; sc[mb] = 0.f;
+    if (mine && mrow < M) {
+      float xs = 0.f, amax = 0.f;
+      for (int bl = 0; bl < nb; ++bl) { xs += s_xs[2 * (mrow * nb + bl) + par]; amax = fmaxf(amax, s_pmax[mrow * nb + bl]); }
+      offs[mb] = 1534.f * xs;
+      sc[mb] = pow2f(scale_exponent(amax));
+    }
   }
   const int hist = history_lane_byteaddr(lane);
+  const size_t slot_floats = (size_t)2 * M * 128;          // one split of one row block
+  float* mypart0 = a.part + ((size_t)rb0 * a.ns + sp) * slot_floats + 16 * w + 8 * (g & 1);
+
   f4 acc[MB][2];
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) { acc[mb][0] = f4{0.f, 0.f, 0.f, 0.f}; acc[mb][1] = f4{0.f, 0.f, 0.f, 0.f}; }
 
-  for (int s0 = 0; s0 < nb; s0 += P) {
+  // ---- main loop: one 128-column block (8 tiles of this wave's strip) per step
+  int cur_r = 0, cur_s = 0;
+  for (int v0 = 0; v0 < total; v0 += P) {
 #pragma unroll
     for (int p = 0; p < P; ++p) {
-      const int s = s0 + p;
-      if (s < nb) {
+      const int v = v0 + p;
+      if (v < total) {
         const StreamRegs<K> cur = buf[p];
-        if (s + P < nb) load_stream<K>(wp + (size_t)(s + P) * STEP_DWORDS, buf[p]);
+        if (v + P < total) prefetch(buf[p]);
         Window<K> win;
         win.build(cur, (uint32_t)__builtin_amdgcn_ds_bpermute(hist, (int)cur.d[K - 1]));
         h8 B0[MB], B1[MB];
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) {
-          const _Float16* bp = xt + boff[mb] + s * 128;
+          const _Float16* bp = xt + boff[mb] + cur_s * 128;
           B0[mb] = *(const h8*)bp;
           B1[mb] = *(const h8*)(bp + 8);
         }
@@ -283,79 +368,79 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
         const h8 A3 = win.template group8<24>();    // row 2q + 1, columns 8..15
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) acc[mb][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A3, B1[mb], acc[mb][1], 0, 0, 0);
-      }
-    }
-  }
 
-  // ---- fold the two tile parities, remove the 1534 offset, undo the activation scale -> this wave's strip partial.
-  // D[i][c] sits in lane c + 16 * (i / 4), register i % 4.  Row pair q is D row q (even tiles, column 2r) plus
-  // D row q + 8 (odd tiles, column 2r + 1): lane (g', c) with g' < 2 and c even adds lane + 33 and then holds rows
-  // 8g' .. 8g' + 7 of the strip for activation row c / 2.
-  // Partials and the arrival counter use agent-scope (write-through / L2-bypassing) accesses, so no cache-wide
-  // writeback or invalidate is needed.
-  float* mypart = a.part + ((size_t)(rb * a.ns + sp) * M) * 128;
-  {
-    const int partner = ((lane + 33) & 63) << 2;
-    const bool keeper = g < 2 && (n16 & 1) == 0;
+        if (++cur_s == nb) {
+          // end of a row block: this wave's strip partials, one per tile parity, with the 1534 offset removed and the
+          // activation scale undone.  Stored with the lowest mantissa bit set (never the all-zero pattern), device
+          // scope (written through), not waited for here.
+          float* dst0 = mypart0 + (size_t)cur_r * a.ns * slot_floats;
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-      const int mrow = mb * 8 + (n16 >> 1);
-      const bool live = keeper && mrow < M;
-      float xs = 0.f, sc = 0.f;
-      if (live) {
-        float amax = 0.f;
-        for (int bl = 0; bl < nb; ++bl) { xs += s_xs[mrow * nb + bl]; amax = fmaxf(amax, s_pmax[mrow * nb + bl]); }
-        const float bound = amax * SQRT128;
-        int e = 0;
-        if (bound > 0.f && bound < 3.0e38f) e = ilogbf(bound) - 13;
-        sc = ldexpf(1.f, e);
-      }
-      float out[8];
+          for (int mb = 0; mb < MB; ++mb) {
+            const int mrow = mb * 8 + (n16 >> 1);
+            if (mine && mrow < M) {
+              uint32_t* dst = (uint32_t*)(dst0 + (size_t)(par * M + mrow) * 128);
 #pragma unroll
-      for (int rr = 0; rr < 2; ++rr)
+              for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const float mine = acc[mb][rr][j];
-          const float other = __uint_as_float((uint32_t)__builtin_amdgcn_ds_bpermute(partner, (int)__float_as_uint(mine)));
-          out[2 * j + rr] = ((mine + other) - 1534.f * xs) * sc;
+                for (int rr = 0; rr < 2; ++rr)
+                  __hip_atomic_store(dst + 2 * j + rr, __float_as_uint((acc[mb][rr][j] - offs[mb]) * sc[mb]) | 1u,
+                                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            acc[mb][0] = f4{0.f, 0.f, 0.f, 0.f}; acc[mb][1] = f4{0.f, 0.f, 0.f, 0.f};
+          }
+          cur_s = 0; ++cur_r;
         }
-      if (live) {
-        float* dst = mypart + mrow * 128 + 16 * w + 8 * g;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) __hip_atomic_store(dst + i, out[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
   }
-  // device-scope stores are acknowledged once written through; wait for every acknowledgement before the barrier
-  // lets thread 0 announce the workgroup (a cache-wide writeback would also do, at many times the cost).
-  // One arrival per workgroup: atomics on one address serialise, so the count is kept as low as possible.
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  __shared__ uint32_t s_old;
-  __syncthreads();
-  if (threadIdx.x == 0) s_old = __hip_atomic_fetch_add(&a.cnt[rb], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  __syncthreads();
-  if (s_old != (uint32_t)(a.ns - 1)) return;
 
-  // ---- last workgroup of the row block: sum the splits in a fixed order, row scale, H128, sv, bias, cast
-  if (threadIdx.x == 0) __hip_atomic_store(&a.cnt[rb], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // ready for the next call
-  const int r0 = rb * 128 + lane, r1 = r0 + 64;
-  const float rs0 = f16_bits_to_float(a.scales[r0]) * a.cbscale, rs1 = f16_bits_to_float(a.scales[r1]) * a.cbscale;
-  const float sg0 = sign_of(a.sv, r0), sg1 = sign_of(a.sv, r1);
-  for (int mrow = w; mrow < M; mrow += WG_WAVES) {
+  // ---- cross-workgroup reduction.  The workspace is all-zero between calls.  Device-scope stores are acknowledged
+  // once written through, so after the wait and the barrier every partial of this workgroup is visible device-wide
+  // (a cache-wide writeback would also do, at many times the cost).
+  //   election by slots:   the workgroup reads every split's slots of a row block; if none is zero all splits have
+  //                        arrived and it finishes the row block.  Several workgroups may see a complete set; they
+  //                        compute bit-identical results (fixed summation order) and store the same values.
+  //   election by counter: one arrival per workgroup and row block; the last one finishes.  Same-address atomics
+  //                        serialise, so this is used only where re-reading the slots would cost more.
+  // Either way the finisher zeroes what it consumed.
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  if (a.by_counter) {
+    if ((int)threadIdx.x < nrb)
+      s_finish[threadIdx.x] = __hip_atomic_fetch_add(&a.cnt[rb0 + threadIdx.x], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                              == (uint32_t)(a.ns - 1);
+    __syncthreads();
+    if ((int)threadIdx.x < nrb && s_finish[threadIdx.x])
+      __hip_atomic_store(&a.cnt[rb0 + threadIdx.x], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+
+  for (int idx = w; idx < nrb * M; idx += WG_WAVES) {
+    const int r = idx / M, mrow = idx - r * M, rb = rb0 + r;
+    if (a.by_counter && !s_finish[r]) continue;
+    const int r0 = rb * 128 + lane, r1 = r0 + 64;
+    const float rs0 = f16_bits_to_float(a.scales[r0]) * a.cbscale, rs1 = f16_bits_to_float(a.scales[r1]) * a.cbscale;
+    const float sg0 = sign_of(a.sv, r0), sg1 = sign_of(a.sv, r1);
+    float b0v = 0.f, b1v = 0.f;
+    if (a.bias != nullptr) { b0v = load_elem(a.bias, a.y_dtype, r0); b1v = load_elem(a.bias, a.y_dtype, r1); }
     float v0 = 0.f, v1 = 0.f;
-    const float* pp = a.part + ((size_t)rb * a.ns * M + mrow) * 128;
-    for (int s = 0; s < a.ns; ++s) {
-      v0 += __hip_atomic_load(pp + (size_t)s * M * 128 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      v1 += __hip_atomic_load(pp + (size_t)s * M * 128 + lane + 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    bool missing = false;
+    uint32_t* pp = (uint32_t*)(a.part + (size_t)rb * a.ns * slot_floats + (size_t)mrow * 128);
+#pragma unroll 8
+    for (int s = 0; s < 2 * a.ns; ++s) {     // slot order: split 0 even, split 0 odd, split 1 even, ...
+      const uint32_t u0 = __hip_atomic_load(pp + (size_t)s * M * 128 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const uint32_t u1 = __hip_atomic_load(pp + (size_t)s * M * 128 + lane + 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      missing |= (u0 == 0u) | (u1 == 0u);
+      v0 += __uint_as_float(u0); v1 += __uint_as_float(u1);
+    }
+    if (__any(missing)) continue;             // some split has not arrived yet: a later workgroup finishes this row
+    for (int s = 0; s < 2 * a.ns; ++s) {      // leave the workspace zero for the next call
+      __hip_atomic_store(pp + (size_t)s * M * 128 + lane, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(pp + (size_t)s * M * 128 + lane + 64, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     v0 *= rs0; v1 *= rs1;
     fwht128_wave(v0, v1, lane);
-    v0 = v0 * INV_SQRT128 * sg0;
-    v1 = v1 * INV_SQRT128 * sg1;
-    if (a.bias != nullptr) {
-      v0 += load_elem(a.bias, a.y_dtype, r0);
-      v1 += load_elem(a.bias, a.y_dtype, r1);
-    }
+    v0 = v0 * INV_SQRT128 * sg0 + b0v;
+    v1 = v1 * INV_SQRT128 * sg1 + b1v;
     store_elem(a.y, a.y_dtype, (size_t)mrow * a.m + r0, v0);
     store_elem(a.y, a.y_dtype, (size_t)mrow * a.m + r1, v1);
   }
@@ -430,37 +515,51 @@ __global__ __launch_bounds__(256) void k_dequant_q(const uint32_t* __restrict__ 
 // ------------------------------------------------------------------------------------------------ host side
 thread_local int g_last_hip_error = 0;
 
-struct Plan { int ns, bps, mb; size_t lds; };
+struct Plan { int ns, bps, rpw, groups, mb, by_counter; size_t lds; };
 
+constexpr int NUM_CU = 256;
+constexpr int MAX_ROW_BLOCKS = 16384;                       // counter region: one word per 128-row block
+inline size_t counters_bytes() { return (size_t)MAX_ROW_BLOCKS * 4; }
+
+// Picks the column split count and the number of row blocks a workgroup walks.  Cost model in microseconds, fitted to
+// kernel traces on MI355X: a compute unit retires one workgroup-step (8 waves x 8 tiles) per ~0.17 us whatever the
+// number of resident workgroups (the decode is VALU-bound); each (row, block) rotation costs a wave ~0.1 us once per
+// workgroup; the slot reads of the election-by-slots protocol grow with ns^2.
 inline bool make_plan(int m, int n, int M, int nsplit, Plan& pl) {
   const int nblk = n / 128, rbs = m / 128;
   pl.mb = M <= 8 ? 1 : (M <= 16 ? 2 : 4);
-  // largest number of 128-column blocks per workgroup that fits the LDS budget
-  int bps_max = 1;
+  int bps_max = 1;     // largest number of 128-column blocks per workgroup that fits the LDS budget
   while (bps_max < nblk && lds_bytes(M, bps_max + 1) <= (size_t)LDS_BUDGET) ++bps_max;
-  int ns;
-  if (nsplit > 0) ns = nsplit;
-  else {
-    // enough workgroups for two per CU, but at least two column blocks each when the matrix allows
-    ns = (512 + rbs - 1) / rbs;
-    if (ns > nblk / 2) ns = nblk / 2;
-    if (ns < 1) ns = 1;
+  double best = 1e30;
+  bool found = false;
+  const int want_ns = nsplit & 0xFFFF, want_rpw = (nsplit >> 16) & 0xFFFF;   // explicit choices (tuning), 0 = search
+  for (int ns = 1; ns <= nblk && ns <= 64; ++ns) {
+    if (want_ns > 0 && ns != want_ns) continue;
+    const int bps = (nblk + ns - 1) / ns;
+    if (bps > bps_max) continue;
+    if ((nblk + bps - 1) / bps != ns) continue;             // this split count is not reachable with equal blocks
+    for (int rpw = 1; rpw <= MAX_RPW && rpw <= rbs; ++rpw) {
+      if (want_rpw > 0 && rpw != want_rpw) continue;
+      const int groups = (rbs + rpw - 1) / rpw;
+      const long wgs = (long)groups * ns;
+      const double rounds = (double)((wgs + NUM_CU - 1) / NUM_CU);
+      const double slot_kb = 2.0 * ns * M * 0.5;            // KB a workgroup reads per row block (election by slots)
+      const int by_counter = (slot_kb * rpw > 64.0) ? 1 : 0;
+      double t = 0.1 * ((M * bps + 7) / 8)                  // rotations
+                 + rounds * rpw * bps * 0.17 * (1.0 + 0.25 * (pl.mb - 1))   // decode steps
+                 + (ns > 1 ? 0.3 : 0.0)
+                 + (by_counter ? 0.4 * ns + 0.8 : 0.02 * slot_kb * rpw);
+      if (bps * ns != nblk) t *= 1.05;                      // ragged last split
+      if (t < best) { best = t; pl.ns = ns; pl.bps = bps; pl.rpw = rpw; pl.groups = groups; pl.by_counter = by_counter; found = true; }
+    }
   }
-  if (ns > nblk) ns = nblk;
-  int bps = (nblk + ns - 1) / ns;
-  if (bps > bps_max) { if (nsplit > 0) return false; bps = bps_max; }
-  ns = (nblk + bps - 1) / bps;
-  pl.ns = ns; pl.bps = bps; pl.lds = lds_bytes(M, bps);
+  if (!found) return false;
+  pl.lds = lds_bytes(M, pl.bps);
   return true;
 }
 
-// fixed-size counter region at the start of the workspace, so that partials of one call can never land on words a
-// later call with a different shape uses as counters
-constexpr int MAX_ROW_BLOCKS = 16384;
-inline size_t counters_bytes() { return (size_t)MAX_ROW_BLOCKS * 4; }
-
 template <int K, int MB> int launch_linear_kmb(const LinearArgs& a, int grid, size_t lds, hipStream_t st) {
-  constexpr int P = K <= 4 ? 4 : (K <= 6 ? 3 : 2);
+  constexpr int P = K <= 4 ? 4 : (K <= 6 ? 3 : 2);   // wave-steps of weights in flight
   auto kern = k_linear<K, MB, P>;
   if (lds > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -523,9 +622,18 @@ size_t htr_workspace_bytes(int m, int n, int K, int M, int nsplit) {
   if (K < 2 || K > 8 || m <= 0 || n <= 0 || m % 128 || n % 128 || m / 128 > MAX_ROW_BLOCKS || M < 1 || M > HTR_MAX_BATCH) return 0;
   Plan pl;
   if (!make_plan(m, n, M, nsplit, pl)) return 0;
-  size_t bytes = counters_bytes();
-  bytes += (size_t)(m / 128) * pl.ns * M * 128 * sizeof(float);
-  return bytes;
+  return counters_bytes() + (size_t)(m / 128) * pl.ns * 2 * M * 128 * sizeof(float);
+}
+
+int htr_linear_plan(int m, int n, int K, int M, int nsplit, int* out6) {
+  if (!out6) return HTR_ERR_NULL;
+  if (K < 2 || K > 8) return HTR_ERR_K;
+  if (m <= 0 || n <= 0 || m % 128 || n % 128 || m / 128 > MAX_ROW_BLOCKS) return HTR_ERR_SHAPE;
+  if (M < 1 || M > HTR_MAX_BATCH) return HTR_ERR_BATCH;
+  Plan pl;
+  if (!make_plan(m, n, M, nsplit, pl)) return HTR_ERR_SPLIT;
+  out6[0] = pl.ns; out6[1] = pl.bps; out6[2] = pl.rpw; out6[3] = pl.groups * pl.ns; out6[4] = pl.by_counter; out6[5] = (int)pl.lds;
+  return HTR_OK;
 }
 
 int htr_linear(const void* qweight, const void* scales, const void* su, const void* sv, const void* x, const void* bias,
@@ -549,9 +657,10 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
   a.x = x; a.bias = bias; a.y = y;
   a.cnt = (uint32_t*)workspace;
   a.part = (float*)((unsigned char*)workspace + counters_bytes());
-  a.m = m; a.n = n; a.M = M; a.ns = pl.ns; a.bps = pl.bps; a.x_dtype = x_dtype; a.y_dtype = y_dtype;
+  a.m = m; a.n = n; a.M = M; a.ns = pl.ns; a.bps = pl.bps; a.rpw = pl.rpw; a.by_counter = pl.by_counter;
+  a.x_dtype = x_dtype; a.y_dtype = y_dtype;
   a.cbscale = htr_cbscale();
-  const int grid = (m / 128) * pl.ns;
+  const int grid = pl.groups * pl.ns;
   hipStream_t st = (hipStream_t)stream;
   HTR_FOR_K(K, return launch_linear_k<KK>(a, pl.mb, grid, pl.lds, st));
   return HTR_OK;

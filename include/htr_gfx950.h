@@ -62,9 +62,17 @@ float htr_cbscale(void);
  * ordered on one stream: kernels leave the counter words zero on exit.
  * Reference: the per-device int32[65536] counter tensor (htr/ops.py:24-28) plus the
  * `part` tensors the extension allocates per call (htr/csrc/htr_kernels.cu:1145).
- * nsplit: 0 = library policy, >0 = explicit split count (as in htr_linear).
+ * nsplit: as in htr_linear.
  */
 size_t htr_workspace_bytes(int m, int n, int K, int M, int nsplit);
+
+/*
+ * The launch plan htr_linear would use: out6 = {column splits, 128-column blocks per split, row blocks per
+ * workgroup, workgroups, 1 if finishers are elected by counter, dynamic LDS bytes}.  No reference counterpart as a
+ * function; it exposes what nsplit_for / fused_nsplit decide there (htr/ops.py:31-45).
+ * nsplit: 0 = library policy; otherwise (row blocks per workgroup << 16) | column splits, either part 0 = search.
+ */
+int htr_linear_plan(int m, int n, int K, int M, int nsplit, int* out6);
 
 /*
  * y[M, m] = x[M, n] @ W^T (+ bias) for an HTR-W1 weight, one fused launch: input sign flip +
@@ -74,7 +82,7 @@ size_t htr_workspace_bytes(int m, int n, int K, int M, int nsplit);
  *   x      [M, n] row-major, x_dtype (bf16 / f16 / f32)
  *   bias   [m] in y_dtype, or NULL
  *   y      [M, m] row-major, y_dtype
- *   nsplit 0 = library policy; >0 = number of column splits to use
+ *   nsplit 0 = library policy; otherwise an explicit plan as in htr_linear_plan (tuning)
  */
 int htr_linear(const void* qweight, const void* scales, const void* su, const void* sv,
                const void* x, const void* bias, void* y,

@@ -37,6 +37,8 @@ def parse():
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying HIP graphs")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample (0 = skip)")
     ap.add_argument("--shapes", action="store_true", help="also time every unfused shape on its own")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 256 MiB device copy, so a counter profile of this command holds a kernel of known traffic")
     return ap.parse_args()
 
 
@@ -89,30 +91,45 @@ def main():
             launch(p)
 
     def make_runner(fn, count):
-        """fn(i) for i in range(count), either eagerly or as `count` single-step HIP graphs."""
+        """Returns run(n): executes fn(0), fn(1), ... fn(n-1) (indices mod count), eagerly or by replaying HIP graphs.
+
+        One graph holds a whole pass over the ring (count calls of fn); single-call graphs serve the remainder, so
+        exactly n calls run whatever n is and the host only issues one replay per ring pass.
+        """
         if args.no_graph:
-            return lambda i: fn(i)
-        graphs = []
+            def run_eager(n):
+                for i in range(n):
+                    fn(i)
+            return run_eager
+        full = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(full):
+            for i in range(count):
+                fn(i)
+        singles = []
         for i in range(count):
             g = torch.cuda.CUDAGraph()
             with torch.cuda.graph(g):
                 fn(i)
-            graphs.append(g)
-        return lambda i: graphs[i % count].replay()
+            singles.append(g)
+
+        def run_graph(n):
+            for _ in range(n // count):
+                full.replay()
+            for i in range(n % count):
+                singles[i].replay()
+        return run_graph
 
     for i in range(ring):      # touch everything once outside any capture
         step(i)
     torch.cuda.synchronize()
     run_step = make_runner(step, ring)
 
-    for i in range(args.warmup):
-        run_step(i)
+    run_step(args.warmup)
     torch.cuda.synchronize()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     e0.record()
-    for i in range(args.steps):
-        run_step(i)
+    run_step(args.steps)
     e1.record()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
@@ -125,13 +142,11 @@ def main():
     def time_shape(plist, reps):
         cnt = len(plist)
         runner = make_runner(lambda i: launch(plist[i % cnt]), cnt)
-        for i in range(cnt):
-            runner(i)
+        runner(cnt)
         torch.cuda.synchronize()
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         a.record()
-        for i in range(reps):
-            runner(i)
+        runner(reps)
         b.record()
         torch.cuda.synchronize()
         return a.elapsed_time(b) * 1e3 / reps      # us per launch
@@ -149,6 +164,14 @@ def main():
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                 "kernel": "k_linear<K=4,MB=1> 28672x4096 (gate_up) batch 1", "us_per_launch": round(dom_us, 3),
                 "algorithmic_bytes_per_launch": dom_bytes}
+
+    if args.calibrate_copy:
+        src = torch.randint(0, 256, (256 << 20,), dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     shapes = None
     if args.shapes:
@@ -192,7 +215,7 @@ def main():
         "config": {"workload": "dense 9B decoder layer, K4 HTR-W1, batch 1, 4 launches/step: qkv 6144x4096 (fused), "
                                "o 4096x4096, gate_up 28672x4096 (fused), down 4096x14336; bf16 x~N(0,1)",
                    "K": K, "batch": 1, "packed_bytes_per_step": layer_bytes, "ring_layers": ring,
-                   "ring_bytes": ring * layer_bytes, "launch": "eager" if args.no_graph else "hip-graph replay, one graph per step"},
+                   "ring_bytes": ring * layer_bytes, "launch": "eager" if args.no_graph else "hip-graph replay, one graph per pass over the ring"},
         "pct_hbm": round(value / HBM_PEAK_GBS * 100, 2),
         "us_per_layer": round(ms_per_step * 1e3, 2),
         "us_per_layer_device_events": round(dev_ms_per_step * 1e3, 2),

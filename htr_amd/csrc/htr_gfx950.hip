@@ -178,6 +178,10 @@ template <int K> struct Window {
 __device__ __forceinline__ int history_lane_byteaddr(int lane) { return ((lane & ~7) | ((lane - 1) & 7)) << 2; }
 
 // ------------------------------------------------------------------------------------------------ fused linear
+// The step space of one linear is (128-row block rb, 128-column block blk), row-major: virtual step v = rb * nblk + blk.
+// It is cut into equal contiguous chunks, one per workgroup, so the workgroup count can be a multiple of the CU count
+// whatever the shape.  A chunk may end inside a row block and continue in the next one; each piece of a row block a
+// chunk covers is a "segment" and yields one partial.
 struct LinearArgs {
   const uint32_t* qw;
   const uint16_t* scales;
@@ -187,23 +191,23 @@ struct LinearArgs {
   const void* bias;
   void* y;
   uint32_t* cnt;    // [m/128] arrival counters (election by counter only); zero on entry and on exit
-  float* part;      // [m/128][ns][2][M][128] split partials per tile parity; all-zero on entry and on exit
+  float* part;      // [workgroups][segmax][2][M][128] partials per segment and tile parity; all-zero on entry and on exit
   int m, n, M;
-  int ns;           // column splits
-  int bps;          // 128-column blocks per split
-  int rpw;          // row blocks per workgroup
-  int by_counter;   // 1: elect the finisher of a row block with an arrival counter; 0: by reading every split's slots
+  int chunk;        // virtual steps per workgroup
+  int segmax;       // partial slots reserved per workgroup
+  int by_counter;   // 1: elect the finisher of a row block with an arrival counter; 0: by reading every contributor's slot
   int x_dtype, y_dtype;
   float cbscale;
 };
 
-constexpr int MAX_RPW = 32;    // row blocks one workgroup may walk
+constexpr int MAX_SEG = 64;    // row-block segments one workgroup may produce
 constexpr int PAIR_REGS = 4;   // (activation row, 128-column block) pairs a wave keeps in registers across the barrier
 
-// LDS layout (dynamic): [xt: (M + 1) rows x row_halves f16][pmax: M * bps f32][xs: M * bps * 2 f32 (per tile parity)]
-__host__ __device__ inline int xt_row_halves(int bps) { return bps * 128 + 8; }   // +8 halves: rows land on different banks
-__host__ __device__ inline size_t lds_bytes(int M, int bps) {
-  return (size_t)(M + 1) * xt_row_halves(bps) * 2 + (size_t)M * bps * 4 * 3;
+// LDS layout (dynamic): [xt: (M + 1) rows x row_halves f16][pmax: M * nbl f32][xs: M * nbl * 2 f32 (per tile parity)]
+// nbl = number of distinct column blocks a chunk touches = min(chunk, n / 128)
+__host__ __device__ inline int xt_row_halves(int nbl) { return nbl * 128 + 8; }   // +8 halves: rows land on different banks
+__host__ __device__ inline size_t lds_bytes(int M, int nbl) {
+  return (size_t)(M + 1) * xt_row_halves(nbl) * 2 + (size_t)M * nbl * 4 * 3;
 }
 
 // power-of-two activation scale 2^e with sqrt(128) * amax / 2^e in (8192, 16384]: |H128 x| / sqrt(128) <= sqrt(128) * max|x|,
@@ -215,25 +219,40 @@ __device__ __forceinline__ int scale_exponent(float amax) {
 }
 __device__ __forceinline__ float pow2f(int e) { return __uint_as_float((uint32_t)(127 + e) << 23); }
 
-template <int K, int MB, int P>
+template <int K> struct DecodedStep { h8 a[4]; };   // MFMA A operands of one step: (row 2q | 2q+1) x (columns 0..7 | 8..15)
+
+template <int K> __device__ __forceinline__ void decode_step(const StreamRegs<K>& r, int hist, DecodedStep<K>& d) {
+  Window<K> win;
+  win.build(r, (uint32_t)__builtin_amdgcn_ds_bpermute(hist, (int)r.d[K - 1]));
+  d.a[0] = win.template group8<0>();
+  d.a[1] = win.template group8<8>();
+  d.a[2] = win.template group8<16>();
+  d.a[3] = win.template group8<24>();
+}
+
+template <int K, int MB, int P, int PRE>
 __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
+  static_assert(PRE <= P, "pre-decoded steps come out of the prefetch registers");
   extern __shared__ __align__(16) unsigned char lds[];
-  __shared__ int s_finish[MAX_RPW];
+  __shared__ int s_finish[MAX_SEG];
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  const int grp = blockIdx.x / a.ns, sp = blockIdx.x - grp * a.ns;
-  const int nblk = a.n >> 7, nt = a.n >> 4, rbs = a.m >> 7;
-  const int b0 = sp * a.bps, nb = min(nblk, b0 + a.bps) - b0;
-  const int rb0 = grp * a.rpw, nrb = min(rbs, rb0 + a.rpw) - rb0;
+  const int nblk = a.n >> 7, rbs = a.m >> 7;
   const int M = a.M;
-  const int rowh = xt_row_halves(a.bps);
+  const int vtotal = rbs * nblk;
+  const int v0 = blockIdx.x * a.chunk, nsteps = min(vtotal, v0 + a.chunk) - v0;
+  const int rb_first = v0 / nblk, c0 = v0 - rb_first * nblk;     // first row block and first column block of the chunk
+  const bool all_blocks = nsteps >= nblk;                        // chunk touches every column block
+  const int nbl = all_blocks ? nblk : nsteps;                    // distinct column blocks; LDS slot of block b:
+  const int rowh = xt_row_halves(min(a.chunk, nblk));            //   b if all_blocks, else (b - c0) mod nblk
 
   _Float16* xt = (_Float16*)lds;
   float* s_pmax = (float*)(lds + (size_t)(M + 1) * rowh * 2);
-  float* s_xs = s_pmax + M * a.bps;
+  float* s_xs = s_pmax + M * min(a.chunk, nblk);
 
-  // ---- input rotation of this split's columns: x~ = f16( H128(su . x) / sqrt(128) / sc ), sc a power of two per row.
-  // Pass 1 loads x (sign applied) and publishes max|x| per (row, block); pass 2 rotates, scales, converts.
-  const int npairs = M * nb;
+  // ---- input rotation of the chunk's column blocks: x~ = f16( H128(su . x) / sqrt(128) / sc ), sc a power of two per
+  // activation row.  Pass 1 loads x (sign applied) and publishes max|x| per (row, block); pass 2 rotates, scales, converts.
+  const int npairs = M * nbl;
+  auto pair_col = [&](int li) { int b = all_blocks ? li : c0 + li; if (b >= nblk) b -= nblk; return b * 128; };
   float xa[PAIR_REGS], xb[PAIR_REGS];
   for (int i = threadIdx.x; i < rowh / 2; i += WG_THREADS) ((uint32_t*)(xt + (size_t)M * rowh))[i] = 0u;   // zero row
 #pragma unroll
@@ -241,28 +260,29 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
     const int pi = w + t * WG_WAVES;
     xa[t] = 0.f; xb[t] = 0.f;
     if (pi < npairs) {
-      const int mrow = pi / nb, bl = pi - mrow * nb, col = (b0 + bl) * 128;
+      const int mrow = pi / nbl, li = pi - mrow * nbl, col = pair_col(li);
       const size_t base = (size_t)mrow * a.n + col;
       xa[t] = load_elem(a.x, a.x_dtype, base + lane) * sign_of(a.su, col + lane);
       xb[t] = load_elem(a.x, a.x_dtype, base + lane + 64) * sign_of(a.su, col + lane + 64);
     }
   }
 
-  // ---- start the weight stream.  The workgroup walks row blocks rb0 .. rb0 + nrb - 1, nb steps each; "virtual
-  // step" v = r * nb + s.  This wave's strip of row block rb0 + r starts at tile row (rb0 + r) * 8 + w.
+  // ---- start the weight stream.  This wave's strip of row block rb is tile row rb * 8 + w; its 8 tiles of column
+  // block blk are 64 * K contiguous dwords; a strip is contiguous over blk, the same strip of the next row block
+  // starts 8 strips later.
   constexpr int STEP_DWORDS = 64 * K;
-  const size_t strip_dwords = (size_t)nt * (8 * K);
-  const uint32_t* wbase = a.qw + ((size_t)(rb0 * 8 + w) * nt + (size_t)8 * b0) * (8 * K) + lane * K;
-  const int total = nrb * nb;
+  const size_t strip_dwords = (size_t)nblk * STEP_DWORDS;
+  const uint32_t* pf_ptr = a.qw + (size_t)(rb_first * 8 + w) * strip_dwords + (size_t)c0 * STEP_DWORDS + lane * K;
+  int pf_blk = c0;
   StreamRegs<K> buf[P];
-  int pf_r = 0, pf_s = 0;                        // prefetch position
   auto prefetch = [&](StreamRegs<K>& dst) {
-    load_stream<K>(wbase + (size_t)pf_r * 8 * strip_dwords + (size_t)pf_s * STEP_DWORDS, dst);
-    if (++pf_s == nb) { pf_s = 0; ++pf_r; }
+    load_stream<K>(pf_ptr, dst);
+    pf_ptr += STEP_DWORDS;
+    if (++pf_blk == nblk) { pf_blk = 0; pf_ptr += 7 * strip_dwords; }
   };
 #pragma unroll
   for (int p = 0; p < P; ++p)
-    if (p < total) prefetch(buf[p]);
+    if (p < nsteps) prefetch(buf[p]);
 
 #pragma unroll
   for (int t = 0; t < PAIR_REGS; ++t) {
@@ -273,39 +293,61 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
     }
   }
   for (int pi = w + PAIR_REGS * WG_WAVES; pi < npairs; pi += WG_WAVES) {   // more pairs than registers: max only, reload later
-    const int mrow = pi / nb, bl = pi - mrow * nb;
-    const size_t base = (size_t)mrow * a.n + (size_t)(b0 + bl) * 128;
+    const int mrow = pi / nbl, li = pi - mrow * nbl;
+    const size_t base = (size_t)mrow * a.n + pair_col(li);
     const float mx = wave_max(fmaxf(fabsf(load_elem(a.x, a.x_dtype, base + lane)), fabsf(load_elem(a.x, a.x_dtype, base + lane + 64))));
     if (lane == 0) s_pmax[pi] = mx;
   }
   __syncthreads();
-  for (int t = 0, pi = w; pi < npairs; ++t, pi += WG_WAVES) {
-    const int mrow = pi / nb, bl = pi - mrow * nb, col = (b0 + bl) * 128;
+  auto rotate_pair = [&](int pi, float va, float vb) {
+    const int mrow = pi / nbl, li = pi - mrow * nbl;
     float amax = 0.f;
-    for (int k = 0; k < nb; ++k) amax = fmaxf(amax, s_pmax[mrow * nb + k]);
+    for (int k = 0; k < nbl; ++k) amax = fmaxf(amax, s_pmax[mrow * nbl + k]);
     const float inv_sc = pow2f(-scale_exponent(amax));
-    float va, vb;
-    if (t < PAIR_REGS) {
-      va = 0.f; vb = 0.f;
-#pragma unroll
-      for (int u = 0; u < PAIR_REGS; ++u) if (u == t) { va = xa[u]; vb = xb[u]; }
-    } else {
-      const size_t base = (size_t)mrow * a.n + col;
-      va = load_elem(a.x, a.x_dtype, base + lane) * sign_of(a.su, col + lane);
-      vb = load_elem(a.x, a.x_dtype, base + lane + 64) * sign_of(a.su, col + lane + 64);
-    }
     va *= inv_sc; vb *= inv_sc;
     fwht128_wave(va, vb, lane);
     const _Float16 ha = (_Float16)(va * INV_SQRT128), hb = (_Float16)(vb * INV_SQRT128);
-    xt[(size_t)mrow * rowh + bl * 128 + lane] = ha;
-    xt[(size_t)mrow * rowh + bl * 128 + lane + 64] = hb;
+    xt[(size_t)mrow * rowh + li * 128 + lane] = ha;
+    xt[(size_t)mrow * rowh + li * 128 + lane + 64] = hb;
     // sum of the rounded x~ per tile parity (element j sits in tile j / 16; lane and lane + 64 share the parity)
     const float hs = (float)ha + (float)hb;
     const bool odd_tile = (lane & 16) != 0;
     const float se = wave_sum(odd_tile ? 0.f : hs), so = wave_sum(odd_tile ? hs : 0.f);
     if (lane == 0) { s_xs[2 * pi] = se; s_xs[2 * pi + 1] = so; }
+  };
+  const bool rotator = w < npairs;      // this wave rotates at least one pair
+  // The rotation is a long chain of dependent instructions that every wave of the workgroup waits for: run it at
+  // raised priority so that decoding waves on the same SIMD do not starve it.
+  __builtin_amdgcn_s_setprio(3);
+#pragma unroll
+  for (int t = 0; t < PAIR_REGS; ++t) {   // unrolled: the chains of a wave's pairs interleave
+    const int pi = w + t * WG_WAVES;
+    if (pi < npairs) rotate_pair(pi, xa[t], xb[t]);
   }
+  for (int pi = w + PAIR_REGS * WG_WAVES; pi < npairs; pi += WG_WAVES) {
+    const int mrow = pi / nbl, li = pi - mrow * nbl, col = pair_col(li);
+    const size_t base = (size_t)mrow * a.n + col;
+    rotate_pair(pi, load_elem(a.x, a.x_dtype, base + lane) * sign_of(a.su, col + lane),
+                load_elem(a.x, a.x_dtype, base + lane + 64) * sign_of(a.su, col + lane + 64));
+  }
+  __builtin_amdgcn_s_setprio(0);
+
+  // ---- decode the first steps into registers.  Waves that rotate nothing do it before the x~ barrier, while the
+  // rotating waves sit in their dependency chains, so the rotation latency is not dead time; rotating waves go to
+  // the barrier at once and decode the same steps after it.
+  const int hist = history_lane_byteaddr(lane);
+  DecodedStep<K> pre[PRE];
+  auto predecode = [&]() {
+#pragma unroll
+    for (int p = 0; p < PRE; ++p)
+      if (p < nsteps) {
+        decode_step<K>(buf[p], hist, pre[p]);
+        if (p + P < nsteps) prefetch(buf[p]);
+      }
+  };
+  if (!rotator) predecode();
   __syncthreads();
+  if (rotator) predecode();
 
   // ---- per-lane constants of the product and of the partial store
   // MFMA operands: row i = lane % 16 = (tile parity h = i / 8, row pair q = i % 8); B column c = lane % 16 carries
@@ -316,80 +358,91 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
   const int g = lane >> 4, n16 = lane & 15;
   const int par = g >> 1;
   const bool mine = (n16 & 1) == par;
-  int boff[MB];            // LDS half-index of this lane's B operand for the first block of the split
-  float offs[MB], sc[MB];  // 1534 * sum(x~) of this lane's (row, parity), and the row's activation scale
+  int boff[MB];      // LDS half-index of this lane's B operand in LDS block 0
+  int xsoff[MB];     // index of this lane's (row, parity) x~ sum in LDS block 0, or -1
+  float sc[MB];      // the row's activation scale
+  float offs[MB];    // running 1534 * sum(x~) over the blocks of the current segment
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
     const int mrow = mb * 8 + (n16 >> 1);
+    const bool live = mine && mrow < M;
     boff[mb] = (mrow < M ? mrow : M) * rowh + 16 * (2 * g + (n16 & 1));
+    xsoff[mb] = live ? 2 * (mrow * nbl) + par : -1;
     offs[mb] = 0.f; sc[mb] = 0.f;
-    if (mine && mrow < M) {
-      float xs = 0.f, amax = 0.f;
-      for (int bl = 0; bl < nb; ++bl) { xs += s_xs[2 * (mrow * nb + bl) + par]; amax = fmaxf(amax, s_pmax[mrow * nb + bl]); }
-      offs[mb] = 1534.f * xs;
+    if (live) {
+      float amax = 0.f;
+      for (int k = 0; k < nbl; ++k) amax = fmaxf(amax, s_pmax[mrow * nbl + k]);
       sc[mb] = pow2f(scale_exponent(amax));
     }
   }
-  const int hist = history_lane_byteaddr(lane);
-  const size_t slot_floats = (size_t)2 * M * 128;          // one split of one row block
-  float* mypart0 = a.part + ((size_t)rb0 * a.ns + sp) * slot_floats + 16 * w + 8 * (g & 1);
+  const size_t slot_floats = (size_t)2 * M * 128;          // one segment: [parity][M][128]
+  float* myslot = a.part + (size_t)blockIdx.x * a.segmax * slot_floats + 16 * w + 8 * (g & 1);
 
   f4 acc[MB][2];
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) { acc[mb][0] = f4{0.f, 0.f, 0.f, 0.f}; acc[mb][1] = f4{0.f, 0.f, 0.f, 0.f}; }
 
-  // ---- main loop: one 128-column block (8 tiles of this wave's strip) per step
-  int cur_r = 0, cur_s = 0;
-  for (int v0 = 0; v0 < total; v0 += P) {
+  int cur_blk = c0, cur_li = all_blocks ? c0 : 0, cur_seg = 0, done = 0;
+  auto consume = [&](const DecodedStep<K>& d) {
+    h8 B0[MB], B1[MB];
 #pragma unroll
-    for (int p = 0; p < P; ++p) {
-      const int v = v0 + p;
-      if (v < total) {
-        const StreamRegs<K> cur = buf[p];
-        if (v + P < total) prefetch(buf[p]);
-        Window<K> win;
-        win.build(cur, (uint32_t)__builtin_amdgcn_ds_bpermute(hist, (int)cur.d[K - 1]));
-        h8 B0[MB], B1[MB];
+    for (int mb = 0; mb < MB; ++mb) {
+      const _Float16* bp = xt + boff[mb] + cur_li * 128;
+      B0[mb] = *(const h8*)bp;
+      B1[mb] = *(const h8*)(bp + 8);
+      if (xsoff[mb] >= 0) offs[mb] += 1534.f * s_xs[xsoff[mb] + 2 * cur_li];
+    }
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb) {
-          const _Float16* bp = xt + boff[mb] + cur_s * 128;
-          B0[mb] = *(const h8*)bp;
-          B1[mb] = *(const h8*)(bp + 8);
+    for (int mb = 0; mb < MB; ++mb) acc[mb][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[0], B0[mb], acc[mb][0], 0, 0, 0);
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) acc[mb][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[1], B1[mb], acc[mb][0], 0, 0, 0);
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) acc[mb][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[2], B0[mb], acc[mb][1], 0, 0, 0);
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) acc[mb][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[3], B1[mb], acc[mb][1], 0, 0, 0);
+    ++done; ++cur_blk; ++cur_li;
+    const bool row_end = cur_blk == nblk;
+    if (row_end || done == nsteps) {
+      // end of a segment: this wave's strip partials, one per tile parity, with the 1534 offset removed and the
+      // activation scale undone.  Stored with the lowest mantissa bit set (never the all-zero pattern), device scope
+      // (written through), not waited for here.
+      float* dst0 = myslot + (size_t)cur_seg * slot_floats;
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        const int mrow = mb * 8 + (n16 >> 1);
+        if (xsoff[mb] >= 0) {
+          uint32_t* dst = (uint32_t*)(dst0 + (size_t)(par * M + mrow) * 128);
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int rr = 0; rr < 2; ++rr)
+              __hip_atomic_store(dst + 2 * j + rr, __float_as_uint((acc[mb][rr][j] - offs[mb]) * sc[mb]) | 1u,
+                                 __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        const h8 A0 = win.template group8<0>();     // row 2q,     columns 0..7 of the lane's tile
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb) acc[mb][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A0, B0[mb], acc[mb][0], 0, 0, 0);
-        const h8 A1 = win.template group8<8>();     // row 2q,     columns 8..15
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb) acc[mb][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A1, B1[mb], acc[mb][0], 0, 0, 0);
-        const h8 A2 = win.template group8<16>();    // row 2q + 1, columns 0..7
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb) acc[mb][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A2, B0[mb], acc[mb][1], 0, 0, 0);
-        const h8 A3 = win.template group8<24>();    // row 2q + 1, columns 8..15
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb) acc[mb][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(A3, B1[mb], acc[mb][1], 0, 0, 0);
+        acc[mb][0] = f4{0.f, 0.f, 0.f, 0.f}; acc[mb][1] = f4{0.f, 0.f, 0.f, 0.f};
+        offs[mb] = 0.f;
+      }
+      ++cur_seg;
+      if (row_end) { cur_blk = 0; if (all_blocks) cur_li = 0; }
+    }
+  };
 
-        if (++cur_s == nb) {
-          // end of a row block: this wave's strip partials, one per tile parity, with the 1534 offset removed and the
-          // activation scale undone.  Stored with the lowest mantissa bit set (never the all-zero pattern), device
-          // scope (written through), not waited for here.
-          float* dst0 = mypart0 + (size_t)cur_r * a.ns * slot_floats;
 #pragma unroll
-          for (int mb = 0; mb < MB; ++mb) {
-            const int mrow = mb * 8 + (n16 >> 1);
-            if (mine && mrow < M) {
-              uint32_t* dst = (uint32_t*)(dst0 + (size_t)(par * M + mrow) * 128);
+  for (int p = 0; p < PRE; ++p)
+    if (p < nsteps) consume(pre[p]);
+
+  // ---- main loop: one 128-column block (8 tiles of this wave's strip) per step; buffer p holds step v with v % P == p
+  for (int vb = PRE; vb < nsteps; vb += P) {
 #pragma unroll
-              for (int j = 0; j < 4; ++j)
-#pragma unroll
-                for (int rr = 0; rr < 2; ++rr)
-                  __hip_atomic_store(dst + 2 * j + rr, __float_as_uint((acc[mb][rr][j] - offs[mb]) * sc[mb]) | 1u,
-                                     __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-            acc[mb][0] = f4{0.f, 0.f, 0.f, 0.f}; acc[mb][1] = f4{0.f, 0.f, 0.f, 0.f};
-          }
-          cur_s = 0; ++cur_r;
-        }
+    for (int pp = 0; pp < P; ++pp) {
+      constexpr int dummy = 0; (void)dummy;
+      const int p = (PRE + pp) % P;
+      const int v = vb + pp;
+      if (v < nsteps) {
+        DecodedStep<K> d;
+        decode_step<K>(buf[p], hist, d);
+        if (v + P < nsteps) prefetch(buf[p]);
+        consume(d);
       }
     }
   }
@@ -397,52 +450,69 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
   // ---- cross-workgroup reduction.  The workspace is all-zero between calls.  Device-scope stores are acknowledged
   // once written through, so after the wait and the barrier every partial of this workgroup is visible device-wide
   // (a cache-wide writeback would also do, at many times the cost).
-  //   election by slots:   the workgroup reads every split's slots of a row block; if none is zero all splits have
-  //                        arrived and it finishes the row block.  Several workgroups may see a complete set; they
-  //                        compute bit-identical results (fixed summation order) and store the same values.
+  //   election by slots:   for each row block it touched the workgroup reads the slots of every contributing chunk;
+  //                        if none is zero all have arrived and it finishes the row block.  Several workgroups may
+  //                        see a complete set; they compute bit-identical results (fixed summation order) and store
+  //                        the same values.
   //   election by counter: one arrival per workgroup and row block; the last one finishes.  Same-address atomics
   //                        serialise, so this is used only where re-reading the slots would cost more.
   // Either way the finisher zeroes what it consumed.
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
+  const int nseg = cur_seg;
   if (a.by_counter) {
-    if ((int)threadIdx.x < nrb)
-      s_finish[threadIdx.x] = __hip_atomic_fetch_add(&a.cnt[rb0 + threadIdx.x], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
-                              == (uint32_t)(a.ns - 1);
+    if ((int)threadIdx.x < nseg) {
+      const int rb = rb_first + threadIdx.x;
+      const int j0 = (rb * nblk) / a.chunk, j1 = (rb * nblk + nblk - 1) / a.chunk;
+      s_finish[threadIdx.x] = __hip_atomic_fetch_add(&a.cnt[rb], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (uint32_t)(j1 - j0);
+    }
     __syncthreads();
-    if ((int)threadIdx.x < nrb && s_finish[threadIdx.x])
-      __hip_atomic_store(&a.cnt[rb0 + threadIdx.x], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if ((int)threadIdx.x < nseg && s_finish[threadIdx.x])
+      __hip_atomic_store(&a.cnt[rb_first + threadIdx.x], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 
-  for (int idx = w; idx < nrb * M; idx += WG_WAVES) {
-    const int r = idx / M, mrow = idx - r * M, rb = rb0 + r;
-    if (a.by_counter && !s_finish[r]) continue;
+  for (int idx = w; idx < nseg * M; idx += WG_WAVES) {
+    const int seg = idx / M, mrow = idx - seg * M, rb = rb_first + seg;
+    if (a.by_counter && !s_finish[seg]) continue;
     const int r0 = rb * 128 + lane, r1 = r0 + 64;
     const float rs0 = f16_bits_to_float(a.scales[r0]) * a.cbscale, rs1 = f16_bits_to_float(a.scales[r1]) * a.cbscale;
     const float sg0 = sign_of(a.sv, r0), sg1 = sign_of(a.sv, r1);
     float b0v = 0.f, b1v = 0.f;
     if (a.bias != nullptr) { b0v = load_elem(a.bias, a.y_dtype, r0); b1v = load_elem(a.bias, a.y_dtype, r1); }
-    float v0 = 0.f, v1 = 0.f;
+    // contributors: chunks j0..j1 overlap row block rb; chunk j holds it in its segment rb - (first row block of j)
+    const int j0 = (rb * nblk) / a.chunk, j1 = (rb * nblk + nblk - 1) / a.chunk;
+    const int sj0 = rb - (j0 * a.chunk) / nblk;              // every later contributor starts inside rb: segment 0
+    float v0s = 0.f, v1s = 0.f;
     bool missing = false;
-    uint32_t* pp = (uint32_t*)(a.part + (size_t)rb * a.ns * slot_floats + (size_t)mrow * 128);
+    auto slot_of = [&](int j) {
+      return (uint32_t*)(a.part + ((size_t)j * a.segmax + (j == j0 ? sj0 : 0)) * slot_floats + (size_t)mrow * 128);
+    };
 #pragma unroll 8
-    for (int s = 0; s < 2 * a.ns; ++s) {     // slot order: split 0 even, split 0 odd, split 1 even, ...
-      const uint32_t u0 = __hip_atomic_load(pp + (size_t)s * M * 128 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const uint32_t u1 = __hip_atomic_load(pp + (size_t)s * M * 128 + lane + 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      missing |= (u0 == 0u) | (u1 == 0u);
-      v0 += __uint_as_float(u0); v1 += __uint_as_float(u1);
+    for (int j = j0; j <= j1; ++j) {
+      const uint32_t* pp = slot_of(j);
+#pragma unroll
+      for (int pr = 0; pr < 2; ++pr) {
+        const uint32_t u0 = __hip_atomic_load(pp + (size_t)pr * M * 128 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t u1 = __hip_atomic_load(pp + (size_t)pr * M * 128 + lane + 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        missing |= (u0 == 0u) | (u1 == 0u);
+        v0s += __uint_as_float(u0); v1s += __uint_as_float(u1);
+      }
     }
-    if (__any(missing)) continue;             // some split has not arrived yet: a later workgroup finishes this row
-    for (int s = 0; s < 2 * a.ns; ++s) {      // leave the workspace zero for the next call
-      __hip_atomic_store(pp + (size_t)s * M * 128 + lane, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_store(pp + (size_t)s * M * 128 + lane + 64, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (__any(missing)) continue;             // some contributor has not arrived yet: a later workgroup finishes this row
+    for (int j = j0; j <= j1; ++j) {          // leave the workspace zero for the next call
+      uint32_t* pp = slot_of(j);
+#pragma unroll
+      for (int pr = 0; pr < 2; ++pr) {
+        __hip_atomic_store(pp + (size_t)pr * M * 128 + lane, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(pp + (size_t)pr * M * 128 + lane + 64, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
     }
-    v0 *= rs0; v1 *= rs1;
-    fwht128_wave(v0, v1, lane);
-    v0 = v0 * INV_SQRT128 * sg0 + b0v;
-    v1 = v1 * INV_SQRT128 * sg1 + b1v;
-    store_elem(a.y, a.y_dtype, (size_t)mrow * a.m + r0, v0);
-    store_elem(a.y, a.y_dtype, (size_t)mrow * a.m + r1, v1);
+    v0s *= rs0; v1s *= rs1;
+    fwht128_wave(v0s, v1s, lane);
+    v0s = v0s * INV_SQRT128 * sg0 + b0v;
+    v1s = v1s * INV_SQRT128 * sg1 + b1v;
+    store_elem(a.y, a.y_dtype, (size_t)mrow * a.m + r0, v0s);
+    store_elem(a.y, a.y_dtype, (size_t)mrow * a.m + r1, v1s);
   }
 }
 
@@ -515,52 +585,62 @@ __global__ __launch_bounds__(256) void k_dequant_q(const uint32_t* __restrict__ 
 // ------------------------------------------------------------------------------------------------ host side
 thread_local int g_last_hip_error = 0;
 
-struct Plan { int ns, bps, rpw, groups, mb, by_counter; size_t lds; };
+struct Plan { int chunk, wgs, segmax, nbl, mb, by_counter; size_t lds; };
 
 constexpr int NUM_CU = 256;
 constexpr int MAX_ROW_BLOCKS = 16384;                       // counter region: one word per 128-row block
 inline size_t counters_bytes() { return (size_t)MAX_ROW_BLOCKS * 4; }
 
-// Picks the column split count and the number of row blocks a workgroup walks.  Cost model in microseconds, fitted to
-// kernel traces on MI355X: a compute unit retires one workgroup-step (8 waves x 8 tiles) per ~0.17 us whatever the
-// number of resident workgroups (the decode is VALU-bound); each (row, block) rotation costs a wave ~0.1 us once per
-// workgroup; the slot reads of the election-by-slots protocol grow with ns^2.
-inline bool make_plan(int m, int n, int M, int nsplit, Plan& pl) {
+inline bool plan_for_chunk(int m, int n, int M, int chunk, Plan& pl) {
   const int nblk = n / 128, rbs = m / 128;
-  pl.mb = M <= 8 ? 1 : (M <= 16 ? 2 : 4);
-  int bps_max = 1;     // largest number of 128-column blocks per workgroup that fits the LDS budget
-  while (bps_max < nblk && lds_bytes(M, bps_max + 1) <= (size_t)LDS_BUDGET) ++bps_max;
-  double best = 1e30;
-  bool found = false;
-  const int want_ns = nsplit & 0xFFFF, want_rpw = (nsplit >> 16) & 0xFFFF;   // explicit choices (tuning), 0 = search
-  for (int ns = 1; ns <= nblk && ns <= 64; ++ns) {
-    if (want_ns > 0 && ns != want_ns) continue;
-    const int bps = (nblk + ns - 1) / ns;
-    if (bps > bps_max) continue;
-    if ((nblk + bps - 1) / bps != ns) continue;             // this split count is not reachable with equal blocks
-    for (int rpw = 1; rpw <= MAX_RPW && rpw <= rbs; ++rpw) {
-      if (want_rpw > 0 && rpw != want_rpw) continue;
-      const int groups = (rbs + rpw - 1) / rpw;
-      const long wgs = (long)groups * ns;
-      const double rounds = (double)((wgs + NUM_CU - 1) / NUM_CU);
-      const double slot_kb = 2.0 * ns * M * 0.5;            // KB a workgroup reads per row block (election by slots)
-      const int by_counter = (slot_kb * rpw > 64.0) ? 1 : 0;
-      double t = 0.1 * ((M * bps + 7) / 8)                  // rotations
-                 + rounds * rpw * bps * 0.17 * (1.0 + 0.25 * (pl.mb - 1))   // decode steps
-                 + (ns > 1 ? 0.3 : 0.0)
-                 + (by_counter ? 0.4 * ns + 0.8 : 0.02 * slot_kb * rpw);
-      if (bps * ns != nblk) t *= 1.05;                      // ragged last split
-      if (t < best) { best = t; pl.ns = ns; pl.bps = bps; pl.rpw = rpw; pl.groups = groups; pl.by_counter = by_counter; found = true; }
-    }
-  }
-  if (!found) return false;
-  pl.lds = lds_bytes(M, pl.bps);
+  const long vtotal = (long)rbs * nblk;
+  if (chunk < 1 || chunk > vtotal) return false;
+  pl.chunk = chunk;
+  pl.wgs = (int)((vtotal + chunk - 1) / chunk);
+  pl.segmax = chunk == 1 ? 1 : (chunk + nblk - 2) / nblk + 1;
+  pl.nbl = chunk < nblk ? chunk : nblk;
+  pl.lds = lds_bytes(M, pl.nbl);
+  if (pl.segmax > MAX_SEG || pl.lds > (size_t)LDS_BUDGET) return false;
+  // bytes a workgroup re-reads when finishers are elected by slots: per segment, every contributor's two parities
+  const int contributors = chunk >= nblk ? 2 : (nblk + chunk - 1) / chunk + 1;
+  const double slot_kb = (double)pl.segmax * contributors * 2 * M * 0.5;
+  pl.by_counter = slot_kb > 96.0 ? 1 : 0;
   return true;
 }
 
+// Picks the chunk length (virtual steps per workgroup) with a cost model in microseconds fitted to chunk-length sweeps
+// on MI355X (K4, batch 1): a fixed latency chain of ~6 us (launch, x fetch, rotation, store acknowledgement, slot reads,
+// output rotation); ~0.8 us per step while every CU holds at most one workgroup, 0.7 us per step and resident
+// workgroup beyond that, plus contention when workgroups share a CU; chunks that do not divide a row of column blocks
+// (or are not whole rows) cost ~35 % more; every extra contributor to a row block adds slot reads.
+inline bool make_plan(int m, int n, int M, int nsplit, Plan& pl) {
+  const int nblk = n / 128, rbs = m / 128;
+  const long vtotal = (long)rbs * nblk;
+  pl.mb = M <= 8 ? 1 : (M <= 16 ? 2 : 4);
+  if (nsplit > 0) return plan_for_chunk(m, n, M, nsplit, pl);      // explicit chunk length (tuning)
+  double best = 1e30;
+  bool found = false;
+  const int max_chunk = (int)(vtotal < 4096 ? vtotal : 4096);
+  for (int chunk = 1; chunk <= max_chunk; ++chunk) {
+    Plan c;
+    c.mb = pl.mb;
+    if (!plan_for_chunk(m, n, M, chunk, c)) continue;
+    const double k = (double)c.wgs / NUM_CU;
+    const double step = (k <= 1.0 ? 0.8 : 0.7 * k) * (1.0 + 0.25 * (pl.mb - 1));
+    const bool aligned = (nblk % chunk == 0) || (chunk % nblk == 0);
+    const int pairs_per_wave = (M * c.nbl + 7) / 8;
+    const int contributors = chunk >= nblk ? 1 : (nblk + chunk - 1) / chunk;
+    const double t = 6.0 + (k > 1.0 ? 1.5 : 0.0) + 0.15 * (pairs_per_wave - 1) + step * chunk * (aligned ? 1.0 : 1.35)
+                     + 0.1 * contributors + (c.by_counter ? 0.4 * contributors + 1.0 : 0.0);
+    if (t < best) { best = t; pl = c; found = true; }
+  }
+  return found;
+}
+
 template <int K, int MB> int launch_linear_kmb(const LinearArgs& a, int grid, size_t lds, hipStream_t st) {
-  constexpr int P = K <= 4 ? 4 : (K <= 6 ? 3 : 2);   // wave-steps of weights in flight
-  auto kern = k_linear<K, MB, P>;
+  constexpr int P = K <= 4 ? 4 : (K <= 6 ? 3 : 2);          // wave-steps of weights in flight
+  constexpr int PRE = MB == 1 ? (P < 4 ? P : 4) : (MB == 2 ? 2 : 1);   // steps decoded ahead of the x~ barrier
+  auto kern = k_linear<K, MB, P, PRE>;
   if (lds > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
@@ -622,7 +702,7 @@ size_t htr_workspace_bytes(int m, int n, int K, int M, int nsplit) {
   if (K < 2 || K > 8 || m <= 0 || n <= 0 || m % 128 || n % 128 || m / 128 > MAX_ROW_BLOCKS || M < 1 || M > HTR_MAX_BATCH) return 0;
   Plan pl;
   if (!make_plan(m, n, M, nsplit, pl)) return 0;
-  return counters_bytes() + (size_t)(m / 128) * pl.ns * 2 * M * 128 * sizeof(float);
+  return counters_bytes() + (size_t)pl.wgs * pl.segmax * 2 * M * 128 * sizeof(float);
 }
 
 int htr_linear_plan(int m, int n, int K, int M, int nsplit, int* out6) {
@@ -632,7 +712,7 @@ int htr_linear_plan(int m, int n, int K, int M, int nsplit, int* out6) {
   if (M < 1 || M > HTR_MAX_BATCH) return HTR_ERR_BATCH;
   Plan pl;
   if (!make_plan(m, n, M, nsplit, pl)) return HTR_ERR_SPLIT;
-  out6[0] = pl.ns; out6[1] = pl.bps; out6[2] = pl.rpw; out6[3] = pl.groups * pl.ns; out6[4] = pl.by_counter; out6[5] = (int)pl.lds;
+  out6[0] = pl.chunk; out6[1] = pl.wgs; out6[2] = pl.segmax; out6[3] = pl.nbl; out6[4] = pl.by_counter; out6[5] = (int)pl.lds;
   return HTR_OK;
 }
 
@@ -657,10 +737,10 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
   a.x = x; a.bias = bias; a.y = y;
   a.cnt = (uint32_t*)workspace;
   a.part = (float*)((unsigned char*)workspace + counters_bytes());
-  a.m = m; a.n = n; a.M = M; a.ns = pl.ns; a.bps = pl.bps; a.rpw = pl.rpw; a.by_counter = pl.by_counter;
+  a.m = m; a.n = n; a.M = M; a.chunk = pl.chunk; a.segmax = pl.segmax; a.by_counter = pl.by_counter;
   a.x_dtype = x_dtype; a.y_dtype = y_dtype;
   a.cbscale = htr_cbscale();
-  const int grid = pl.groups * pl.ns;
+  const int grid = pl.wgs;
   hipStream_t st = (hipStream_t)stream;
   HTR_FOR_K(K, return launch_linear_k<KK>(a, pl.mb, grid, pl.lds, st));
   return HTR_OK;

@@ -128,10 +128,15 @@ def test_bf16_output_within_one_ulp(dev, oracle):
     y = ops.linear(x.to(dev), *d).float().cpu()
     y32 = ops.linear_f32out(x.to(dev), *d).cpu()
     assert torch.equal(y, y32.bfloat16().float())            # the cast is round-to-nearest-even of the f32 result
-    ref = torch.from_numpy(_ref(oracle, qw, sc, su, sv, x))
+    ref = torch.from_numpy(_ref(oracle, qw, sc, su, sv, x)).float()
     want = ref.bfloat16().float()
-    ulp = want.abs() * 2.0 ** -7 + 1e-30
-    assert bool(torch.all((y - want).abs() <= ulp))
+    # the f32 result carries up to REL_TOL * max|ref| of error (measured 2e-4), so "one bf16 ulp of bf16(y_ref)" can only
+    # hold where an ulp is larger than that: elements above 1/8 of the largest magnitude
+    big = ref.abs() >= 0.125 * ref.abs().max()
+    ulp = torch.maximum(want.abs(), ref.abs()) * 2.0 ** -7
+    assert int(big.sum()) > 20
+    assert bool(torch.all((y - want).abs()[big] <= ulp[big]))
+    assert float((y - ref).abs().max()) <= float(ref.abs().max()) * (2.0 ** -8 + REL_TOL)
 
 
 def test_large_activations_do_not_overflow(dev, oracle):

@@ -1,0 +1,147 @@
+"""CPU-only checks of the boundary: the C ABI library loads and exports what include/htr_gfx950.h declares, argument
+validation returns the documented codes before anything touches a GPU, the launch planner is sane, and the Python
+operator layer mirrors the reference's htr.ops surface (htr/ops.py:69-122 of the reference)."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def L():
+    from htr_amd import _native, build
+    if not os.path.exists(_native.LIB_PATH):
+        build.build()
+    return _native.lib()
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "htr_gfx950.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(htr_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(L):
+    from htr_amd import _native
+    names = _declared_functions()
+    assert {"htr_linear", "htr_decode_raw", "htr_dequant_q", "htr_workspace_bytes", "htr_linear_plan"} <= set(names)
+    for n in names:
+        assert hasattr(L, n), n
+    assert set(_native.SIGNATURES) == set(names)          # the ctypes table binds exactly the header
+
+
+def test_constants(L, oracle):
+    assert L.htr_abi_version() >= 1
+    assert np.float32(L.htr_cbscale()) == np.float32(oracle.c_cbscale())
+    from htr_amd import wire
+    assert wire.cbscale() == oracle.c_cbscale()
+    assert L.htr_strerror(0) == b"ok" and b"K" in L.htr_strerror(2)
+
+
+def test_validation_codes_without_gpu(L):
+    p = ctypes.c_void_p(0x1000)                # never dereferenced: every case below fails validation first
+    ok_ws = ctypes.c_void_p(0x100000)
+    call = lambda **kw: L.htr_linear(kw.get("qw", p), p, p, p, p, None, kw.get("y", p), kw.get("m", 256), kw.get("n", 256),
+                                     kw.get("K", 4), kw.get("M", 1), kw.get("xd", 0), kw.get("yd", 0), kw.get("ns", 0),
+                                     kw.get("ws", ok_ws), kw.get("wsb", 1 << 30), None)
+    assert call(qw=None) == 1
+    assert call(K=1) == 2 and call(K=9) == 2
+    assert call(m=200) == 3 and call(n=0) == 3
+    assert call(M=0) == 4 and call(M=33) == 4
+    assert call(xd=3) == 5 and call(yd=-1) == 5
+    assert call(ws=None) == 6 and call(wsb=16) == 6 and call(ws=ctypes.c_void_p(0x100010)) == 6
+    assert call(qw=ctypes.c_void_p(0x1004)) == 7
+    assert call(ns=100000) == 9
+    assert L.htr_decode_raw(None, p, 8, 4, None) == 1 and L.htr_decode_raw(p, p, 8, 1, None) == 2
+    assert L.htr_dequant_q(p, p, None, 8, 8, 4, None) == 1 and L.htr_dequant_q(p, p, p, 0, 8, 4, None) == 3
+    assert L.htr_workspace_bytes(256, 256, 9, 1, 0) == 0
+
+
+@pytest.mark.parametrize("m,n", [(128, 128), (256, 384), (4096, 4096), (1024, 4096), (6144, 4096), (14336, 4096),
+                                 (28672, 4096), (4096, 14336), (152064, 4096), (1408, 2048), (2048, 1408)])
+@pytest.mark.parametrize("M", [1, 2, 8, 9, 16, 32])
+def test_launch_plan_is_consistent(L, m, n, M):
+    out = (ctypes.c_int * 6)()
+    assert L.htr_linear_plan(m, n, 4, M, 0, out) == 0
+    chunk, wgs, segmax, nbl, by_counter, lds = list(out)
+    nblk, rbs = n // 128, m // 128
+    assert chunk >= 1 and (wgs - 1) * chunk < rbs * nblk <= wgs * chunk          # chunks tile the step space exactly
+    assert nbl == min(chunk, nblk) and lds <= 64 * 1024
+    assert segmax >= 1 and (chunk <= 1 or segmax >= (chunk + nblk - 2) // nblk + 1)
+    need = L.htr_workspace_bytes(m, n, 4, M, 0)
+    assert need >= 65536 + wgs * segmax * 2 * M * 128 * 4
+    # an explicit chunk length is honoured
+    assert L.htr_linear_plan(m, n, 4, M, 1, out) == 0 or M * 128 * 2 > 60000
+    if out[0] == 1:
+        assert out[1] == rbs * nblk
+
+
+def test_wire_helpers_match_oracle(oracle):
+    from htr_amd import wire
+    signs = torch.tensor([1., -1., 1., -1., 1., -1., 1., -1.])
+    assert wire.pack_signs(signs).item() == 170                                  # tests/test_release.py:40-43 of the reference
+    assert torch.equal(wire.unpack_signs(wire.pack_signs(signs), 8), signs)
+    g = torch.Generator().manual_seed(4)
+    words = torch.randint(-(2 ** 31), 2 ** 31, (5, 32), dtype=torch.int32, generator=g)
+    st = torch.from_numpy(oracle.c_unpack_states(words.numpy(), 4).astype(np.int64))
+    assert torch.equal(wire.pack_states(st, 4), words)
+    assert torch.equal(wire.gen_values(st), torch.from_numpy(oracle.np_gen_values(st.numpy())))
+    assert wire.payload_bytes(4096, 14336, 4) == 29370624 and wire.payload_bytes(152064, 4096, 4) == 311750720
+    a = wire.synth_linear(256, 128, 3, 7)
+    b = wire.synth_linear(256, 128, 3, 7)
+    assert all(torch.equal(x, y) for x, y in zip(a, b))
+    assert tuple(a[0].shape) == (16, 8, 24) and a[1].dtype == torch.float16 and a[2].numel() == 16 and a[3].numel() == 32
+    assert wire.check_shapes(*a) == (256, 128, 3)
+    with pytest.raises(RuntimeError):
+        wire.check_shapes(a[0][:, :, :8].contiguous(), a[1], a[2], a[3])        # K = 1
+    with pytest.raises(RuntimeError):
+        wire.check_shapes(a[0][:15], a[1][:240], a[2], a[3][:30])               # m = 240, not a multiple of 128
+    with pytest.raises(RuntimeError):
+        wire.check_shapes(a[0], a[1].float(), a[2], a[3])
+
+
+def test_operator_surface_on_cpu():
+    from htr_amd import ops, wire
+    qw, sc, su, sv = wire.synth_linear(256, 128, 4, 1)
+    # M == 0 short-circuits before any device work (htr/ops.py:73-74 of the reference)
+    y = ops.linear(torch.zeros(0, 128, dtype=torch.bfloat16), qw, sc, su, sv)
+    assert tuple(y.shape) == (0, 256) and y.dtype == torch.bfloat16
+    y = ops.linear(torch.zeros(2, 0, 128, dtype=torch.float16), qw, sc, su, sv)
+    assert tuple(y.shape) == (2, 0, 256) and y.dtype == torch.float16
+    with pytest.raises(RuntimeError):                                          # no CPU implementation, by design
+        ops.linear(torch.zeros(1, 128, dtype=torch.bfloat16), qw, sc, su, sv)
+    with pytest.raises(RuntimeError):
+        ops.linear(torch.zeros(1, 256, dtype=torch.bfloat16), qw, sc, su, sv)  # wrong input width
+    with pytest.raises(KeyError):
+        ops.linear(torch.zeros(1, 128, dtype=torch.float64), qw, sc, su, sv)   # same as the reference's dtype map
+    # custom op registered under the reference's name and schema, with a fake implementation
+    op = torch.ops.htr.linear.default
+    schema = str(op._schema)
+    assert schema.startswith("htr::linear(Tensor x2, Tensor qweight, Tensor scales, Tensor su, Tensor sv, Tensor? bias) -> Tensor")
+    meta = [t.to("meta") for t in (torch.zeros(3, 128, dtype=torch.bfloat16), qw, sc, su, sv)]
+    out = op(*meta, None)
+    assert out.device.type == "meta" and tuple(out.shape) == (3, 256) and out.dtype == torch.bfloat16
+
+
+def test_missing_library_raises(monkeypatch):
+    from htr_amd import _native
+    monkeypatch.setattr(_native, "_lib", None)
+    monkeypatch.setattr(_native, "LIB_PATH", "/nonexistent/libhtr_gfx950.so")
+    with pytest.raises(_native.NativeLibraryMissing):
+        _native.lib()
+
+
+def test_product_never_imports_the_oracle():
+    bad = []
+    for dirpath, _, files in os.walk(os.path.join(ROOT, "htr_amd")):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp")):
+                text = open(os.path.join(dirpath, f)).read()
+                if re.search(r"^\s*(from|import)\s+oracle\b", text, flags=re.M) or "libhtr_oracle" in text:
+                    bad.append(f)
+    assert bad == []

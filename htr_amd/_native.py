@@ -27,6 +27,7 @@ SIGNATURES = {
     "htr_linear": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
     "htr_decode_raw": (_i, [_vp, _vp, _i64, _i, _vp]),
     "htr_dequant_q": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
+    "htr_dequant_w": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
 }
 
 

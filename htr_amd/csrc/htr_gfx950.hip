@@ -582,6 +582,60 @@ __global__ __launch_bounds__(256) void k_dequant_q(const uint32_t* __restrict__ 
   });
 }
 
+// ------------------------------------------------------------------------------------------------ original-basis W
+// W = Sv . Ho . Q . Hi . Su as bf16 [m, n] (htr/wire.py:105-113 of the reference), one workgroup per 128x128 block:
+// decode the 64 tiles into LDS as float32 (row scale * CBSCALE applied), H128 down the columns (Ho), H128 along the
+// rows (Hi), signs, 1/128, round to bf16.  The row pass is last so that the stores are row-contiguous.
+constexpr int DQW_LD = 129;   // LDS leading dimension in floats: odd, so column walks hit distinct banks
+
+template <int K>
+__global__ __launch_bounds__(512) void k_dequant_w(const uint32_t* __restrict__ qw, const uint16_t* __restrict__ scales,
+                                                   const uint8_t* __restrict__ su, const uint8_t* __restrict__ sv,
+                                                   uint16_t* __restrict__ W, int nt, float cbscale) {
+  extern __shared__ __align__(16) unsigned char lds[];
+  float* blk = (float*)lds;                                  // [128][DQW_LD]
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int bj = blockIdx.x, bi = blockIdx.y;                // 128-column block, 128-row block
+  const int n = nt * 16;
+  // thread = (tile in block, row pair q): 64 tiles x 8 = 512 threads; a tile's 8 threads are consecutive lanes
+  {
+    const int t64 = threadIdx.x >> 3, q = threadIdx.x & 7;
+    const int ti = t64 >> 3, tj = t64 & 7;                   // tile row / column inside the block
+    const size_t tile = (size_t)(bi * 8 + ti) * nt + (size_t)bj * 8 + tj;
+    StreamRegs<K> r;
+    load_stream<K>(qw + tile * (8 * K) + q * K, r);
+    Window<K> win;
+    win.build(r, (uint32_t)__builtin_amdgcn_ds_bpermute(history_lane_byteaddr(lane), (int)r.d[K - 1]));
+    const int row0 = ti * 16 + 2 * q;
+    const float s0 = f16_bits_to_float(scales[bi * 128 + row0]) * cbscale;
+    const float s1 = f16_bits_to_float(scales[bi * 128 + row0 + 1]) * cbscale;
+    float* o0 = blk + row0 * DQW_LD + tj * 16;
+    float* o1 = o0 + DQW_LD;
+    ForEach32<K, 0>::run(win, [&](int u, int v) {
+      if (u < 16) o0[u] = (float)v * s0; else o1[u - 16] = (float)v * s1;
+    });
+  }
+  __syncthreads();
+  // Ho: transform every column (wave w takes columns w, w + 8, ...; lane holds rows lane and lane + 64)
+  for (int c = w; c < 128; c += 8) {
+    float a = blk[lane * DQW_LD + c], b = blk[(lane + 64) * DQW_LD + c];
+    fwht128_wave(a, b, lane);
+    blk[lane * DQW_LD + c] = a;
+    blk[(lane + 64) * DQW_LD + c] = b;
+  }
+  __syncthreads();
+  // Hi along every row, then signs and 1/128 (both rotations' 1/sqrt(128)), bf16 store
+  const float su0 = sign_of(su, bj * 128 + lane), su1 = sign_of(su, bj * 128 + lane + 64);
+  for (int r = w; r < 128; r += 8) {
+    float a = blk[r * DQW_LD + lane], b = blk[r * DQW_LD + lane + 64];
+    fwht128_wave(a, b, lane);
+    const float sg = sign_of(sv, bi * 128 + r) * (1.0f / 128.0f);
+    uint16_t* dst = W + (size_t)(bi * 128 + r) * n + (size_t)bj * 128;
+    dst[lane] = float_to_bf16_bits(a * sg * su0);
+    dst[lane + 64] = float_to_bf16_bits(b * sg * su1);
+  }
+}
+
 // ------------------------------------------------------------------------------------------------ host side
 thread_local int g_last_hip_error = 0;
 
@@ -755,6 +809,31 @@ int htr_decode_raw(const void* qweight, void* out_i16, int64_t ntiles, int K, vo
   hipStream_t st = (hipStream_t)stream;
   HTR_FOR_K(K, hipLaunchKernelGGL(k_decode_raw<KK>, dim3((unsigned)blocks), dim3(256), 0, st, (const uint32_t*)qweight,
                                   (int16_t*)out_i16, ntiles));
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
+  return HTR_OK;
+}
+
+int htr_dequant_w(const void* qweight, const void* scales, const void* su, const void* sv, void* out_bf16, int m, int n,
+                  int K, void* stream) {
+  if (!qweight || !scales || !su || !sv || !out_bf16) return HTR_ERR_NULL;
+  if (K < 2 || K > 8) return HTR_ERR_K;
+  if (m <= 0 || n <= 0 || m % 128 || n % 128 || m / 128 > 65535) return HTR_ERR_SHAPE;
+  if (((uintptr_t)qweight & 15) || ((uintptr_t)out_bf16 & 1) || ((uintptr_t)scales & 1)) return HTR_ERR_ALIGN;
+  hipStream_t st = (hipStream_t)stream;
+  const dim3 grid(n / 128, m / 128);
+  const size_t lds = (size_t)128 * DQW_LD * sizeof(float);
+  const float cb = htr_cbscale();
+#define HTR_LAUNCH_DQW(KK_)                                                                                              \
+  {                                                                                                                      \
+    auto kern = k_dequant_w<KK_>;                                                                                        \
+    hipError_t e0 = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);       \
+    if (e0 != hipSuccess) { g_last_hip_error = (int)e0; return HTR_ERR_LAUNCH; }                                         \
+    hipLaunchKernelGGL(kern, grid, dim3(512), lds, st, (const uint32_t*)qweight, (const uint16_t*)scales,                \
+                       (const uint8_t*)su, (const uint8_t*)sv, (uint16_t*)out_bf16, n / 16, cb);                         \
+  }
+  HTR_FOR_K(K, HTR_LAUNCH_DQW(KK));
+#undef HTR_LAUNCH_DQW
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
   return HTR_OK;

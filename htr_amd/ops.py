@@ -17,8 +17,12 @@ _DTYPE_CODE = {torch.bfloat16: _native.BF16, torch.float16: _native.F16, torch.f
 # One launch takes up to this many activation rows; longer inputs are cut into chunks that each
 # re-read the packed weight (the reference does the same in 8-row chunks, htr/ops.py:77-88).
 LAUNCH_MAX_M = _native.MAX_BATCH
-# explicit column-split count for experiments; 0 = library policy
+# explicit chunk length (steps per workgroup) for experiments; 0 = library policy
 NSPLIT = int(os.environ.get("HTR_NSPLIT", "0"))
+# Above this many activation rows the weight is dequantized once to the original basis (bf16) and a library GEMM does
+# the product, as the reference does for prefill (HTR_PREFILL="w", htr/ops.py:52-54,89-93); up to it, the fused
+# decode kernel runs in launches of LAUNCH_MAX_M rows (the reference's HTR_GEMV_LOOP_MAX, htr/ops.py:59-61).
+GEMV_LOOP_MAX = int(os.environ.get("HTR_GEMV_LOOP_MAX", "64"))
 
 _WORKSPACES = {}
 
@@ -69,6 +73,12 @@ def _linear_impl(x2, qweight, scales, su, sv, bias, out_dtype=None):
             raise RuntimeError("HTR-W1 tensors must be contiguous and on the device of x")
     if bias is not None and (bias.dtype != out_dtype or bias.numel() != m or bias.device != x2.device):
         raise RuntimeError("bias must be [m] in the output dtype on the device of x")
+    if M > GEMV_LOOP_MAX:
+        W = dequant_w(qweight, scales, su, sv)
+        if x2.dtype != torch.bfloat16:
+            W = W.to(x2.dtype)
+        y = torch.nn.functional.linear(x2, W, None if bias is None else bias.to(x2.dtype))
+        return y if y.dtype == out_dtype else y.to(out_dtype)
     y = torch.empty((M, m), dtype=out_dtype, device=x2.device)
     code = _DTYPE_CODE[out_dtype]
     with torch.cuda.device(x2.device):
@@ -113,6 +123,19 @@ def decode_raw(qweight):
     with torch.cuda.device(qweight.device):
         st = torch.cuda.current_stream(qweight.device).cuda_stream
         _native.check(_native.lib().htr_decode_raw(qweight.data_ptr(), out.data_ptr(), ntiles, K, st))
+    return out
+
+
+def dequant_w(qweight, scales, su, sv):
+    """Original-basis W bfloat16 [m, n] = Sv.Ho.Q.Hi.Su (dequant_w of the reference extension; wire.dequant on the CPU)."""
+    m, n, K = wire.check_shapes(qweight, scales, su, sv)
+    if not qweight.is_cuda or not all(t.is_contiguous() and t.device == qweight.device for t in (qweight, scales, su, sv)):
+        raise RuntimeError("dequant_w wants contiguous tensors on one ROCm device")
+    out = torch.empty((m, n), dtype=torch.bfloat16, device=qweight.device)
+    with torch.cuda.device(qweight.device):
+        st = torch.cuda.current_stream(qweight.device).cuda_stream
+        _native.check(_native.lib().htr_dequant_w(qweight.data_ptr(), scales.data_ptr(), su.data_ptr(), sv.data_ptr(),
+                                                  out.data_ptr(), m, n, K, st))
     return out
 
 

@@ -73,6 +73,37 @@ def test_dequant_q_bit_exact(dev, oracle, K):
     assert got.dtype == np.float32 and np.array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
+@pytest.mark.parametrize("K", [2, 3, 4, 5, 7])
+def test_dequant_w_original_basis(dev, oracle, K):
+    from htr_amd import ops, wire
+    print(f"dequant_w K={K}", flush=True)
+    qw, sc, su, sv = wire.synth_linear(384, 256, K, 300 + K)
+    got = ops.dequant_w(*[t.to(dev) for t in (qw, sc, su, sv)])
+    assert got.dtype == torch.bfloat16 and tuple(got.shape) == (384, 256)
+    ref = torch.from_numpy(oracle.c_dequant_w(qw.numpy(), sc.numpy(), su.numpy(), sv.numpy()))      # float64
+    g = got.float().cpu().double()
+    # bf16 rounding (2^-9 relative) of a value computed with float32 butterflies (error ~1e-6 of the block's scale)
+    assert float((g - ref).abs().max()) <= float(ref.abs().max()) * 2.0 ** -8
+    err = (g - ref).abs()
+    assert bool(torch.all(err <= ref.abs() * 2.0 ** -8 + float(ref.abs().max()) * 4e-6))
+    # orthogonal rotations preserve the Frobenius norm of Q
+    Q = torch.from_numpy(oracle.c_dequant_q(qw.numpy(), sc.numpy())).double()
+    assert abs(float(g.norm() / Q.norm()) - 1.0) < 2e-3
+
+
+def test_prefill_path_dequant_then_gemm(dev, oracle):
+    from htr_amd import ops
+    print("prefill M=96", flush=True)
+    qw, sc, su, sv, x = _case(512, 384, 4, 96, 808)
+    bias = torch.randn(512, generator=torch.Generator().manual_seed(2)).bfloat16()
+    assert 96 > ops.GEMV_LOOP_MAX
+    y = ops.linear(x.to(dev), *[t.to(dev) for t in (qw, sc, su, sv)], bias.to(dev))
+    assert y.dtype == torch.bfloat16 and tuple(y.shape) == (96, 512)
+    ref = _ref(oracle, qw, sc, su, sv, x, bias)
+    # bf16 weights and bf16 output: compare at bf16 resolution of the largest magnitudes
+    assert _rel(y.float().cpu().numpy(), ref) <= 2.0 ** -6
+
+
 @pytest.mark.parametrize("K", [2, 3, 4, 5])
 @pytest.mark.parametrize("M", [1, 2, 3, 4, 8])
 @pytest.mark.parametrize("shape", [(256, 384), (1024, 4096), (4096, 1024)])

@@ -193,6 +193,10 @@ struct LinearArgs {
   uint32_t* cnt;    // [m/128] arrival counters (election by counter only); zero on entry and on exit
   float* part;      // [workgroups][segmax][2][M][128] partials per segment and tile parity; all-zero on entry and on exit
   int m, n, M;
+  const _Float16* xt_g;   // pre-rotated activations [M][n] f16 (only when prerot)
+  const float* xs_g;      // their per-(row, block, tile parity) sums [M][n/128][2]
+  const float* sc_g;      // per-row activation scale [M]
+  int prerot;             // 1: x~ was produced by k_rotate; 0: this kernel rotates its own column blocks
   int chunk;        // virtual steps per workgroup
   int segmax;       // partial slots reserved per workgroup
   int by_counter;   // 1: elect the finisher of a row block with an arrival counter; 0: by reading every contributor's slot
@@ -205,7 +209,11 @@ constexpr int PAIR_REGS = 4;   // (activation row, 128-column block) pairs a wav
 
 // LDS layout (dynamic): [xt: (M + 1) rows x row_halves f16][pmax: M * nbl f32][xs: M * nbl * 2 f32 (per tile parity)]
 // nbl = number of distinct column blocks a chunk touches = min(chunk, n / 128)
-__host__ __device__ inline int xt_row_halves(int nbl) { return nbl * 128 + 8; }   // +8 halves: rows land on different banks
+// One rotated 128-column block is stored as [columns 0..7 of tiles 0..7][columns 8..15 of tiles 0..7] (2 x 64 halves), and
+// rows are padded by 16 halves: the 16-byte B-operand reads of 8 consecutive lanes (4 activation rows x 2 tile parities)
+// then cover 128 contiguous-mod-128 bytes, i.e. every LDS bank once.
+__host__ __device__ inline int xt_row_halves(int nbl) { return nbl * 128 + 16; }
+__device__ __forceinline__ int xt_slot(int j) { return ((j >> 3) & 1) * 64 + (j >> 4) * 8 + (j & 7); }   // element j of a block
 __host__ __device__ inline size_t lds_bytes(int M, int nbl) {
   return (size_t)(M + 1) * xt_row_halves(nbl) * 2 + (size_t)M * nbl * 4 * 3;
 }
@@ -219,6 +227,39 @@ __device__ __forceinline__ int scale_exponent(float amax) {
 }
 __device__ __forceinline__ float pow2f(int e) { return __uint_as_float((uint32_t)(127 + e) << 23); }
 
+// Rotation of all activation rows ahead of the linear kernel (used from 3 rows up, where every workgroup rotating its
+// own column blocks would repeat the same work hundreds of times): one workgroup per row.
+__global__ __launch_bounds__(WG_THREADS) void k_rotate(const void* __restrict__ x, const uint8_t* __restrict__ su, int n, int x_dtype,
+                                                       _Float16* __restrict__ xt_g, float* __restrict__ xs_g, float* __restrict__ sc_g) {
+  __shared__ float s_max[WG_WAVES];
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, mrow = blockIdx.x, nblk = n >> 7;
+  const size_t row = (size_t)mrow * n;
+  float mx = 0.f;
+  for (int i = threadIdx.x; i < n; i += WG_THREADS) mx = fmaxf(mx, fabsf(load_elem(x, x_dtype, row + i)));
+  mx = wave_max(mx);
+  if (lane == 0) s_max[w] = mx;
+  __syncthreads();
+  float amax = 0.f;
+#pragma unroll
+  for (int k = 0; k < WG_WAVES; ++k) amax = fmaxf(amax, s_max[k]);
+  const int e = scale_exponent(amax);
+  const float inv_sc = pow2f(-e);
+  if (threadIdx.x == 0) sc_g[mrow] = pow2f(e);
+  for (int blk = w; blk < nblk; blk += WG_WAVES) {
+    const int col = blk * 128;
+    float va = load_elem(x, x_dtype, row + col + lane) * sign_of(su, col + lane) * inv_sc;
+    float vb = load_elem(x, x_dtype, row + col + lane + 64) * sign_of(su, col + lane + 64) * inv_sc;
+    fwht128_wave(va, vb, lane);
+    const _Float16 ha = (_Float16)(va * INV_SQRT128), hb = (_Float16)(vb * INV_SQRT128);
+    xt_g[row + col + lane] = ha;
+    xt_g[row + col + lane + 64] = hb;
+    const float hs = (float)ha + (float)hb;
+    const bool odd_tile = (lane & 16) != 0;
+    const float se = wave_sum(odd_tile ? 0.f : hs), so = wave_sum(odd_tile ? hs : 0.f);
+    if (lane == 0) { xs_g[((size_t)mrow * nblk + blk) * 2] = se; xs_g[((size_t)mrow * nblk + blk) * 2 + 1] = so; }
+  }
+}
+
 template <int K> struct DecodedStep { h8 a[4]; };   // MFMA A operands of one step: (row 2q | 2q+1) x (columns 0..7 | 8..15)
 
 template <int K> __device__ __forceinline__ void decode_step(const StreamRegs<K>& r, int hist, DecodedStep<K>& d) {
@@ -230,7 +271,7 @@ template <int K> __device__ __forceinline__ void decode_step(const StreamRegs<K>
   d.a[3] = win.template group8<24>();
 }
 
-template <int K, int MB, int P, int PRE>
+template <int K, int MB, int P, int PRE, bool PREROT>
 __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
   static_assert(PRE <= P, "pre-decoded steps come out of the prefetch registers");
   extern __shared__ __align__(16) unsigned char lds[];
@@ -254,12 +295,27 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
   const int npairs = M * nbl;
   auto pair_col = [&](int li) { int b = all_blocks ? li : c0 + li; if (b >= nblk) b -= nblk; return b * 128; };
   float xa[PAIR_REGS], xb[PAIR_REGS];
+  constexpr bool prerot = PREROT;   // x~ comes from k_rotate instead of being rotated here
   for (int i = threadIdx.x; i < rowh / 2; i += WG_THREADS) ((uint32_t*)(xt + (size_t)M * rowh))[i] = 0u;   // zero row
+  // with pre-rotated activations: 16-byte pieces of this chunk's x~ slice, issued before the weight stream
+  constexpr int COPY_REGS = 4;
+  u4 cp[COPY_REGS];
+  const int ncopy = npairs * 16;                 // 16 pieces of 8 halves per (row, block) pair
+  if constexpr (prerot) {
+#pragma unroll
+    for (int t = 0; t < COPY_REGS; ++t) {
+      const int ci = threadIdx.x + t * WG_THREADS;
+      if (ci < ncopy) {
+        const int pi = ci >> 4, mrow = pi / nbl, li = pi - mrow * nbl;
+        cp[t] = *(const u4*)(a.xt_g + (size_t)mrow * a.n + pair_col(li) + (ci & 15) * 8);
+      }
+    }
+  }
 #pragma unroll
   for (int t = 0; t < PAIR_REGS; ++t) {     // x first: loads return in order, and x heads the longest dependency chain
     const int pi = w + t * WG_WAVES;
     xa[t] = 0.f; xb[t] = 0.f;
-    if (pi < npairs) {
+    if (!prerot && pi < npairs) {
       const int mrow = pi / nbl, li = pi - mrow * nbl, col = pair_col(li);
       const size_t base = (size_t)mrow * a.n + col;
       xa[t] = load_elem(a.x, a.x_dtype, base + lane) * sign_of(a.su, col + lane);
@@ -284,6 +340,8 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
   for (int p = 0; p < P; ++p)
     if (p < nsteps) prefetch(buf[p]);
 
+  const bool rotator = !prerot && w < npairs;      // this wave rotates at least one pair
+  if constexpr (!prerot) {
 #pragma unroll
   for (int t = 0; t < PAIR_REGS; ++t) {
     const int pi = w + t * WG_WAVES;
@@ -307,15 +365,14 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
     va *= inv_sc; vb *= inv_sc;
     fwht128_wave(va, vb, lane);
     const _Float16 ha = (_Float16)(va * INV_SQRT128), hb = (_Float16)(vb * INV_SQRT128);
-    xt[(size_t)mrow * rowh + li * 128 + lane] = ha;
-    xt[(size_t)mrow * rowh + li * 128 + lane + 64] = hb;
+    xt[(size_t)mrow * rowh + li * 128 + xt_slot(lane)] = ha;
+    xt[(size_t)mrow * rowh + li * 128 + xt_slot(lane + 64)] = hb;
     // sum of the rounded x~ per tile parity (element j sits in tile j / 16; lane and lane + 64 share the parity)
     const float hs = (float)ha + (float)hb;
     const bool odd_tile = (lane & 16) != 0;
     const float se = wave_sum(odd_tile ? 0.f : hs), so = wave_sum(odd_tile ? hs : 0.f);
     if (lane == 0) { s_xs[2 * pi] = se; s_xs[2 * pi + 1] = so; }
   };
-  const bool rotator = w < npairs;      // this wave rotates at least one pair
   // The rotation is a long chain of dependent instructions that every wave of the workgroup waits for: run it at
   // raised priority so that decoding waves on the same SIMD do not starve it.
   __builtin_amdgcn_s_setprio(3);
@@ -332,6 +389,26 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
   }
   __builtin_amdgcn_s_setprio(0);
 
+  } else {
+    // copy the slice into LDS; sums per (row, block, parity) come with it
+#pragma unroll
+    for (int t = 0; t < COPY_REGS; ++t) {
+      const int ci = threadIdx.x + t * WG_THREADS;
+      if (ci < ncopy) {
+        const int pi = ci >> 4, mrow = pi / nbl, li = pi - mrow * nbl;
+        *(u4*)(xt + (size_t)mrow * rowh + li * 128 + (ci & 1) * 64 + ((ci & 15) >> 1) * 8) = cp[t];
+      }
+    }
+    for (int ci = threadIdx.x + COPY_REGS * WG_THREADS; ci < ncopy; ci += WG_THREADS) {
+      const int pi = ci >> 4, mrow = pi / nbl, li = pi - mrow * nbl;
+      *(u4*)(xt + (size_t)mrow * rowh + li * 128 + (ci & 1) * 64 + ((ci & 15) >> 1) * 8) =
+          *(const u4*)(a.xt_g + (size_t)mrow * a.n + pair_col(li) + (ci & 15) * 8);
+    }
+    for (int i = threadIdx.x; i < npairs * 2; i += WG_THREADS) {
+      const int pi = i >> 1, mrow = pi / nbl, li = pi - mrow * nbl;
+      s_xs[i] = a.xs_g[((size_t)mrow * nblk + (pair_col(li) >> 7)) * 2 + (i & 1)];
+    }
+  }
   // ---- decode the first steps into registers.  Waves that rotate nothing do it before the x~ barrier, while the
   // rotating waves sit in their dependency chains, so the rotation latency is not dead time; rotating waves go to
   // the barrier at once and decode the same steps after it.
@@ -366,13 +443,16 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
   for (int mb = 0; mb < MB; ++mb) {
     const int mrow = mb * 8 + (n16 >> 1);
     const bool live = mine && mrow < M;
-    boff[mb] = (mrow < M ? mrow : M) * rowh + 16 * (2 * g + (n16 & 1));
+    boff[mb] = (mrow < M ? mrow : M) * rowh + 8 * (2 * g + (n16 & 1));
     xsoff[mb] = live ? 2 * (mrow * nbl) + par : -1;
     offs[mb] = 0.f; sc[mb] = 0.f;
     if (live) {
-      float amax = 0.f;
-      for (int k = 0; k < nbl; ++k) amax = fmaxf(amax, s_pmax[mrow * nbl + k]);
-      sc[mb] = pow2f(scale_exponent(amax));
+      if constexpr (prerot) sc[mb] = a.sc_g[mrow];
+      else {
+        float amax = 0.f;
+        for (int k = 0; k < nbl; ++k) amax = fmaxf(amax, s_pmax[mrow * nbl + k]);
+        sc[mb] = pow2f(scale_exponent(amax));
+      }
     }
   }
   const size_t slot_floats = (size_t)2 * M * 128;          // one segment: [parity][M][128]
@@ -389,7 +469,7 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
     for (int mb = 0; mb < MB; ++mb) {
       const _Float16* bp = xt + boff[mb] + cur_li * 128;
       B0[mb] = *(const h8*)bp;
-      B1[mb] = *(const h8*)(bp + 8);
+      B1[mb] = *(const h8*)(bp + 64);
       if (xsoff[mb] >= 0) offs[mb] += 1534.f * s_xs[xsoff[mb] + 2 * cur_li];
     }
 #pragma unroll
@@ -639,7 +719,15 @@ __global__ __launch_bounds__(512) void k_dequant_w(const uint32_t* __restrict__ 
 // ------------------------------------------------------------------------------------------------ host side
 thread_local int g_last_hip_error = 0;
 
-struct Plan { int chunk, wgs, segmax, nbl, mb, by_counter; size_t lds; };
+struct Plan { int chunk, wgs, segmax, nbl, mb, by_counter, prerot; size_t lds; };
+
+constexpr int PREROT_MIN_M = 6;   // from this many rows on the activations are rotated once by k_rotate
+// The pre-rotated activations live in a fixed region between the counters and the partial slots: partial slots must be
+// all-zero between calls, and no call may leave other data where a later call of another shape expects such slots.
+constexpr size_t PREROT_REGION = (size_t)4 << 20;
+inline size_t align256(size_t v) { return (v + 255) / 256 * 256; }
+// bytes of the pre-rotated activations, their block sums and the row scales
+inline size_t prerot_bytes(int n, int M) { return align256((size_t)M * n * 2) + align256((size_t)M * (n / 128) * 8) + align256((size_t)M * 4); }
 
 constexpr int NUM_CU = 256;
 constexpr int MAX_ROW_BLOCKS = 16384;                       // counter region: one word per 128-row block
@@ -659,6 +747,7 @@ inline bool plan_for_chunk(int m, int n, int M, int chunk, Plan& pl) {
   const int contributors = chunk >= nblk ? 2 : (nblk + chunk - 1) / chunk + 1;
   const double slot_kb = (double)pl.segmax * contributors * 2 * M * 0.5;
   pl.by_counter = slot_kb > 96.0 ? 1 : 0;
+  pl.prerot = (M >= PREROT_MIN_M && prerot_bytes(n, M) <= PREROT_REGION) ? 1 : 0;
   return true;
 }
 
@@ -682,7 +771,7 @@ inline bool make_plan(int m, int n, int M, int nsplit, Plan& pl) {
     const double k = (double)c.wgs / NUM_CU;
     const double step = (k <= 1.0 ? 0.8 : 0.7 * k) * (1.0 + 0.25 * (pl.mb - 1));
     const bool aligned = (nblk % chunk == 0) || (chunk % nblk == 0);
-    const int pairs_per_wave = (M * c.nbl + 7) / 8;
+    const int pairs_per_wave = c.prerot ? 1 : (M * c.nbl + 7) / 8;
     const int contributors = chunk >= nblk ? 1 : (nblk + chunk - 1) / chunk;
     const double t = 6.0 + (k > 1.0 ? 1.5 : 0.0) + 0.15 * (pairs_per_wave - 1) + step * chunk * (aligned ? 1.0 : 1.35)
                      + 0.1 * contributors + (c.by_counter ? 0.4 * contributors + 1.0 : 0.0);
@@ -691,10 +780,9 @@ inline bool make_plan(int m, int n, int M, int nsplit, Plan& pl) {
   return found;
 }
 
-template <int K, int MB> int launch_linear_kmb(const LinearArgs& a, int grid, size_t lds, hipStream_t st) {
+template <int K, int MB, int PRE, bool PREROT> int launch_linear_v(const LinearArgs& a, int grid, size_t lds, hipStream_t st) {
   constexpr int P = K <= 4 ? 4 : (K <= 6 ? 3 : 2);          // wave-steps of weights in flight
-  constexpr int PRE = MB == 1 ? (P < 4 ? P : 4) : (MB == 2 ? 2 : 1);   // steps decoded ahead of the x~ barrier
-  auto kern = k_linear<K, MB, P, PRE>;
+  auto kern = k_linear<K, MB, P, (PRE < P ? PRE : P), PREROT>;
   if (lds > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
@@ -704,12 +792,18 @@ template <int K, int MB> int launch_linear_kmb(const LinearArgs& a, int grid, si
   if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
   return HTR_OK;
 }
-template <int K> int launch_linear_k(const LinearArgs& a, int mb, int grid, size_t lds, hipStream_t st) {
+// Steps decoded ahead of the x~ barrier: deep (more registers, fewer resident waves) only for short chunks, where the
+// prologue latency is a large part of the kernel; long chunks prefer occupancy.
+template <int K, bool PREROT> int launch_linear_kr(const LinearArgs& a, int mb, int grid, size_t lds, hipStream_t st) {
+  const bool deep = a.chunk <= 8;
   switch (mb) {
-    case 1: return launch_linear_kmb<K, 1>(a, grid, lds, st);
-    case 2: return launch_linear_kmb<K, 2>(a, grid, lds, st);
-    default: return launch_linear_kmb<K, 4>(a, grid, lds, st);
+    case 1: return deep ? launch_linear_v<K, 1, 4, PREROT>(a, grid, lds, st) : launch_linear_v<K, 1, 1, PREROT>(a, grid, lds, st);
+    case 2: return deep ? launch_linear_v<K, 2, 2, PREROT>(a, grid, lds, st) : launch_linear_v<K, 2, 1, PREROT>(a, grid, lds, st);
+    default: return launch_linear_v<K, 4, 1, PREROT>(a, grid, lds, st);
   }
+}
+template <int K> int launch_linear_k(const LinearArgs& a, int mb, int grid, size_t lds, hipStream_t st) {
+  return a.prerot ? launch_linear_kr<K, true>(a, mb, grid, lds, st) : launch_linear_kr<K, false>(a, mb, grid, lds, st);
 }
 
 #define HTR_FOR_K(K, EXPR)                 \
@@ -756,7 +850,7 @@ size_t htr_workspace_bytes(int m, int n, int K, int M, int nsplit) {
   if (K < 2 || K > 8 || m <= 0 || n <= 0 || m % 128 || n % 128 || m / 128 > MAX_ROW_BLOCKS || M < 1 || M > HTR_MAX_BATCH) return 0;
   Plan pl;
   if (!make_plan(m, n, M, nsplit, pl)) return 0;
-  return counters_bytes() + (size_t)pl.wgs * pl.segmax * 2 * M * 128 * sizeof(float);
+  return counters_bytes() + PREROT_REGION + (size_t)pl.wgs * pl.segmax * 2 * M * 128 * sizeof(float);
 }
 
 int htr_linear_plan(int m, int n, int K, int M, int nsplit, int* out6) {
@@ -790,12 +884,25 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
   a.qw = (const uint32_t*)qweight; a.scales = (const uint16_t*)scales; a.su = (const uint8_t*)su; a.sv = (const uint8_t*)sv;
   a.x = x; a.bias = bias; a.y = y;
   a.cnt = (uint32_t*)workspace;
-  a.part = (float*)((unsigned char*)workspace + counters_bytes());
+  unsigned char* wsp = (unsigned char*)workspace + counters_bytes();
+  a.prerot = pl.prerot; a.xt_g = nullptr; a.xs_g = nullptr; a.sc_g = nullptr;
+  if (pl.prerot) {
+    a.xt_g = (const _Float16*)wsp;
+    a.xs_g = (const float*)(wsp + align256((size_t)M * n * 2));
+    a.sc_g = (const float*)(wsp + align256((size_t)M * n * 2) + align256((size_t)M * (n / 128) * 8));
+  }
+  a.part = (float*)(wsp + PREROT_REGION);
   a.m = m; a.n = n; a.M = M; a.chunk = pl.chunk; a.segmax = pl.segmax; a.by_counter = pl.by_counter;
   a.x_dtype = x_dtype; a.y_dtype = y_dtype;
   a.cbscale = htr_cbscale();
   const int grid = pl.wgs;
   hipStream_t st = (hipStream_t)stream;
+  if (pl.prerot) {
+    hipLaunchKernelGGL(k_rotate, dim3(M), dim3(WG_THREADS), 0, st, x, (const uint8_t*)su, n, x_dtype, (_Float16*)a.xt_g,
+                       (float*)a.xs_g, (float*)a.sc_g);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
+  }
   HTR_FOR_K(K, return launch_linear_k<KK>(a, pl.mb, grid, pl.lds, st));
   return HTR_OK;
 }

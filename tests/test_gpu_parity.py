@@ -220,3 +220,68 @@ def test_full_size_shapes(dev, oracle, K, m, n):
     # linearity in x, a size-independent property: f(2x) == 2 f(x) exactly (power-of-two scaling)
     y2 = ops.linear_f32out((x * 2).to(dev), *d).cpu().numpy()
     assert np.array_equal(y2, 2 * y)
+
+
+# ---- BASELINE configs 4 and 5 as parity cases
+@pytest.mark.parametrize("K,M,m,n", [(3, 8, 14336, 4096), (4, 16, 14336, 4096), (4, 32, 4096, 14336), (3, 32, 14336, 4096),
+                                     (4, 8, 4096, 14336)])
+def test_small_batch_gemm_shapes(dev, oracle, K, M, m, n):
+    from htr_amd import ops
+    print(f"small-batch K={K} M={M} {m}x{n}", flush=True)
+    qw, sc, su, sv, x = _case(m, n, K, M, 4000 + 13 * K + M)
+    y = ops.linear_f32out(x.to(dev), *[t.to(dev) for t in (qw, sc, su, sv)]).cpu().numpy()
+    ref = _ref(oracle, qw, sc, su, sv, x)
+    for r in range(M):
+        assert _rel(y[r], ref[r]) <= REL_TOL, (r, _rel(y[r], ref[r]))
+
+
+def test_moe_expert_stack_top6_of_64(dev, oracle):
+    """64 experts (gate/up 1408x2048, down 2048x1408, K4), top-6 routing of 16 tokens; each active expert is a pair of
+    packed linears (the reference has no MoE kernel: docs/ADAPTERS.md:19).  Eight experts are materialised; the routing
+    ids are folded onto them so that the composition, token gathering and accumulation are all exercised."""
+    from htr_amd import ops, wire
+    print("moe expert stack", flush=True)
+    E, T, TOP, H, F = 8, 16, 6, 2048, 1408
+    g = torch.Generator().manual_seed(20261125 + 5000)
+    probs = torch.softmax(torch.randn(T, 64, generator=g), dim=-1)
+    w, ids = torch.topk(probs, TOP, dim=-1)
+    ids = ids % E
+    x = torch.randn(T, H, generator=g).bfloat16()
+    experts = []
+    for e in range(E):
+        gu = wire.synth_linear(2 * F, H, 4, 7000 + e)            # gate and up fused along the output dim (shared su)
+        dn = wire.synth_linear(H, F, 4, 7100 + e)
+        experts.append((gu, dn))
+    y = torch.zeros(T, H, dtype=torch.float32, device=dev)
+    y_ref = np.zeros((T, H))
+    xd = x.to(dev)
+    for e, (gu, dn) in enumerate(experts):
+        tok, slot = torch.nonzero(ids == e, as_tuple=True)
+        if tok.numel() == 0:
+            continue
+        wt = w[tok, slot]
+        gud = [t.to(dev) for t in gu]
+        dnd = [t.to(dev) for t in dn]
+        h2 = ops.linear_f32out(xd[tok.to(dev)].contiguous(), *gud)
+        h = (torch.nn.functional.silu(h2[:, :F]) * h2[:, F:]).bfloat16()
+        out = ops.linear_f32out(h.contiguous(), *dnd)
+        y.index_add_(0, tok.to(dev), out * wt.to(dev)[:, None])
+        # same composition on the CPU oracle, with the same bf16 rounding of the hidden activation
+        r2 = oracle.c_linear(x[tok].float().numpy(), *[t.numpy() for t in gu])
+        rh = torch.from_numpy(r2).float()
+        rh = (torch.nn.functional.silu(rh[:, :F]) * rh[:, F:]).bfloat16().float().numpy()
+        ro = oracle.c_linear(rh, *[t.numpy() for t in dn])
+        np.add.at(y_ref, tok.numpy(), ro * wt.numpy().astype(np.float64)[:, None])
+    got = y.cpu().numpy()
+    # two chained linears with a bf16 rounding between them: the first stage's 2e-4 error moves some hidden values by
+    # one bf16 ulp, so the end-to-end bar is looser than one linear's
+    assert _rel(got, y_ref) <= 4e-3, _rel(got, y_ref)
+
+
+def test_lm_head_shape(dev, oracle):
+    from htr_amd import ops
+    print("lm_head 152064x4096", flush=True)
+    qw, sc, su, sv, x = _case(152064, 4096, 4, 1, 20261125 + 5001)
+    y = ops.linear_f32out(x.to(dev), *[t.to(dev) for t in (qw, sc, su, sv)]).cpu().numpy()
+    ref = _ref(oracle, qw, sc, su, sv, x)
+    assert _rel(y, ref) <= REL_TOL, _rel(y, ref)

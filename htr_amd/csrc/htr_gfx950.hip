@@ -276,7 +276,9 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
   static_assert(PRE <= P, "pre-decoded steps come out of the prefetch registers");
   extern __shared__ __align__(16) unsigned char lds[];
   __shared__ int s_finish[MAX_SEG];
-  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));   // wave index, provably uniform: keeps the
+                                                                           // strip addressing on the scalar unit
   const int nblk = a.n >> 7, rbs = a.m >> 7;
   const int M = a.M;
   const int vtotal = rbs * nblk;
@@ -328,11 +330,12 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
   // starts 8 strips later.
   constexpr int STEP_DWORDS = 64 * K;
   const size_t strip_dwords = (size_t)nblk * STEP_DWORDS;
-  const uint32_t* pf_ptr = a.qw + (size_t)(rb_first * 8 + w) * strip_dwords + (size_t)c0 * STEP_DWORDS + lane * K;
+  const uint32_t* pf_ptr = a.qw + (size_t)(rb_first * 8 + w) * strip_dwords + (size_t)c0 * STEP_DWORDS;   // uniform
+  const int lane_dwords = lane * K;
   int pf_blk = c0;
   StreamRegs<K> buf[P];
   auto prefetch = [&](StreamRegs<K>& dst) {
-    load_stream<K>(pf_ptr, dst);
+    load_stream<K>(pf_ptr + lane_dwords, dst);
     pf_ptr += STEP_DWORDS;
     if (++pf_blk == nblk) { pf_blk = 0; pf_ptr += 7 * strip_dwords; }
   };
@@ -422,9 +425,11 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
         if (p + P < nsteps) prefetch(buf[p]);
       }
   };
-  if (!rotator) predecode();
+  // (when most waves rotate, the few that do not would only delay the barrier by decoding first)
+  const bool early = !rotator && npairs <= WG_WAVES / 2;
+  if (early) predecode();
   __syncthreads();
-  if (rotator) predecode();
+  if (!early) predecode();
 
   // ---- per-lane constants of the product and of the partial store
   // MFMA operands: row i = lane % 16 = (tile parity h = i / 8, row pair q = i % 8); B column c = lane % 16 carries

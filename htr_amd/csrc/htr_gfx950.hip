@@ -111,6 +111,16 @@ __device__ __forceinline__ float wave_sum(float v) {
   halves16(v, e, o); v = e + o;
   halves32(v, e, o); return e + o;
 }
+// sums of v over the lanes with (lane & 16) == 0 and over those with (lane & 16) != 0, in every lane
+__device__ __forceinline__ void wave_sum_by_row_parity(float v, float& even_rows, float& odd_rows) {
+  v += lane_xor_dpp<1>(v); v += lane_xor_dpp<2>(v); v += lane_xor_dpp<4>(v); v += lane_xor_dpp<8>(v);   // per 16-lane row
+  float lo, hi;
+  halves32(v, lo, hi);          // lo: rows 0/1 as seen from the lane's position in its half, hi: rows 2/3
+  const float s = lo + hi;      // row 0 + row 2 in even rows' lanes, row 1 + row 3 in odd rows' lanes
+  float e, o;
+  halves16(s, e, o);
+  even_rows = e; odd_rows = o;
+}
 __device__ __forceinline__ float wave_max(float v) {
   v = fmaxf(v, lane_xor_dpp<1>(v)); v = fmaxf(v, lane_xor_dpp<2>(v)); v = fmaxf(v, lane_xor_dpp<4>(v)); v = fmaxf(v, lane_xor_dpp<8>(v));
   float e, o;
@@ -207,7 +217,7 @@ struct LinearArgs {
 constexpr int MAX_SEG = 64;    // row-block segments one workgroup may produce
 constexpr int PAIR_REGS = 4;   // (activation row, 128-column block) pairs a wave keeps in registers across the barrier
 
-// LDS layout (dynamic): [xt: (M + 1) rows x row_halves f16][pmax: M * nbl f32][xs: M * nbl * 2 f32 (per tile parity)]
+// LDS layout (dynamic): [xt: (M + 1) rows x row_halves f16][pmax: M * nbl f32][xs: M * nbl * 2 f32 (per tile parity)][sc: M f32]
 // nbl = number of distinct column blocks a chunk touches = min(chunk, n / 128)
 // One rotated 128-column block is stored as [columns 0..7 of tiles 0..7][columns 8..15 of tiles 0..7] (2 x 64 halves), and
 // rows are padded by 16 halves: the 16-byte B-operand reads of 8 consecutive lanes (4 activation rows x 2 tile parities)
@@ -215,7 +225,7 @@ constexpr int PAIR_REGS = 4;   // (activation row, 128-column block) pairs a wav
 __host__ __device__ inline int xt_row_halves(int nbl) { return nbl * 128 + 16; }
 __device__ __forceinline__ int xt_slot(int j) { return ((j >> 3) & 1) * 64 + (j >> 4) * 8 + (j & 7); }   // element j of a block
 __host__ __device__ inline size_t lds_bytes(int M, int nbl) {
-  return (size_t)(M + 1) * xt_row_halves(nbl) * 2 + (size_t)M * nbl * 4 * 3;
+  return (size_t)(M + 1) * xt_row_halves(nbl) * 2 + (size_t)M * nbl * 4 * 3 + (size_t)M * 4;
 }
 
 // power-of-two activation scale 2^e with sqrt(128) * amax / 2^e in (8192, 16384]: |H128 x| / sqrt(128) <= sqrt(128) * max|x|,
@@ -253,9 +263,8 @@ __global__ __launch_bounds__(WG_THREADS) void k_rotate(const void* __restrict__ 
     const _Float16 ha = (_Float16)(va * INV_SQRT128), hb = (_Float16)(vb * INV_SQRT128);
     xt_g[row + col + lane] = ha;
     xt_g[row + col + lane + 64] = hb;
-    const float hs = (float)ha + (float)hb;
-    const bool odd_tile = (lane & 16) != 0;
-    const float se = wave_sum(odd_tile ? 0.f : hs), so = wave_sum(odd_tile ? hs : 0.f);
+    float se, so;
+    wave_sum_by_row_parity((float)ha + (float)hb, se, so);
     if (lane == 0) { xs_g[((size_t)mrow * nblk + blk) * 2] = se; xs_g[((size_t)mrow * nblk + blk) * 2 + 1] = so; }
   }
 }
@@ -291,6 +300,7 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
   _Float16* xt = (_Float16*)lds;
   float* s_pmax = (float*)(lds + (size_t)(M + 1) * rowh * 2);
   float* s_xs = s_pmax + M * min(a.chunk, nblk);
+  float* s_sc = s_xs + 2 * M * min(a.chunk, nblk);     // activation scale per row
 
   // ---- input rotation of the chunk's column blocks: x~ = f16( H128(su . x) / sqrt(128) / sc ), sc a power of two per
   // activation row.  Pass 1 loads x (sign applied) and publishes max|x| per (row, block); pass 2 rotates, scales, converts.
@@ -360,20 +370,25 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
     if (lane == 0) s_pmax[pi] = mx;
   }
   __syncthreads();
+  // max|x| of activation row mrow over the chunk's blocks: lanes read the per-block maxima, one wave reduction
+  auto row_amax = [&](int mrow) {
+    float v = 0.f;
+    for (int k = lane; k < nbl; k += 64) v = fmaxf(v, s_pmax[mrow * nbl + k]);
+    return wave_max(v);
+  };
   auto rotate_pair = [&](int pi, float va, float vb) {
     const int mrow = pi / nbl, li = pi - mrow * nbl;
-    float amax = 0.f;
-    for (int k = 0; k < nbl; ++k) amax = fmaxf(amax, s_pmax[mrow * nbl + k]);
-    const float inv_sc = pow2f(-scale_exponent(amax));
+    const int e = scale_exponent(row_amax(mrow));
+    const float inv_sc = pow2f(-e);
+    if (li == 0 && lane == 0) s_sc[mrow] = pow2f(e);
     va *= inv_sc; vb *= inv_sc;
     fwht128_wave(va, vb, lane);
     const _Float16 ha = (_Float16)(va * INV_SQRT128), hb = (_Float16)(vb * INV_SQRT128);
     xt[(size_t)mrow * rowh + li * 128 + xt_slot(lane)] = ha;
     xt[(size_t)mrow * rowh + li * 128 + xt_slot(lane + 64)] = hb;
     // sum of the rounded x~ per tile parity (element j sits in tile j / 16; lane and lane + 64 share the parity)
-    const float hs = (float)ha + (float)hb;
-    const bool odd_tile = (lane & 16) != 0;
-    const float se = wave_sum(odd_tile ? 0.f : hs), so = wave_sum(odd_tile ? hs : 0.f);
+    float se, so;
+    wave_sum_by_row_parity((float)ha + (float)hb, se, so);
     if (lane == 0) { s_xs[2 * pi] = se; s_xs[2 * pi + 1] = so; }
   };
   // The rotation is a long chain of dependent instructions that every wave of the workgroup waits for: run it at
@@ -453,11 +468,7 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
     offs[mb] = 0.f; sc[mb] = 0.f;
     if (live) {
       if constexpr (prerot) sc[mb] = a.sc_g[mrow];
-      else {
-        float amax = 0.f;
-        for (int k = 0; k < nbl; ++k) amax = fmaxf(amax, s_pmax[mrow * nbl + k]);
-        sc[mb] = pow2f(scale_exponent(amax));
-      }
+      else sc[mb] = s_sc[mrow];
     }
   }
   const size_t slot_floats = (size_t)2 * M * 128;          // one segment: [parity][M][128]

@@ -349,11 +349,12 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
     pf_ptr += STEP_DWORDS;
     if (++pf_blk == nblk) { pf_blk = 0; pf_ptr += 7 * strip_dwords; }
   };
-#pragma unroll
-  for (int p = 0; p < P; ++p)
-    if (p < nsteps) prefetch(buf[p]);
-
   const bool rotator = !prerot && w < npairs;      // this wave rotates at least one pair
+  if constexpr (prerot) {
+#pragma unroll
+    for (int p = 0; p < P; ++p)
+      if (p < nsteps) prefetch(buf[p]);
+  }
   if constexpr (!prerot) {
 #pragma unroll
   for (int t = 0; t < PAIR_REGS; ++t) {
@@ -363,6 +364,13 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
       if (lane == 0) s_pmax[pi] = mx;
     }
   }
+  // The weight stream starts only now, after x has arrived: when every wave of the chip bursts its first weight loads
+  // at once, an x load issued just before them takes about twice as long, and x heads the critical chain, while the
+  // rotation below hides the weight latency anyway.
+  asm volatile("" ::: "memory");
+#pragma unroll
+  for (int p = 0; p < P; ++p)
+    if (p < nsteps) prefetch(buf[p]);
   for (int pi = w + PAIR_REGS * WG_WAVES; pi < npairs; pi += WG_WAVES) {   // more pairs than registers: max only, reload later
     const int mrow = pi / nbl, li = pi - mrow * nbl;
     const size_t base = (size_t)mrow * a.n + pair_col(li);
@@ -796,9 +804,21 @@ inline bool make_plan(int m, int n, int M, int nsplit, Plan& pl) {
   return found;
 }
 
+// The dispatcher places workgroups wherever resources allow, not evenly: with 512 equal workgroups some CUs receive
+// three and others one, and the kernel ends with the most loaded CU.  Requesting 1/k of a CU's 160 KB of LDS per
+// workgroup (k = workgroups per CU when spread evenly) makes exactly k fit, so the spread is even.
+constexpr size_t CU_LDS_BYTES = 160 * 1024;
+inline size_t balanced_lds_request(size_t needed, int grid) {
+  const int k = (grid + NUM_CU - 1) / NUM_CU;
+  if (k > 4) return needed;
+  const size_t share = (CU_LDS_BYTES / k) / 1024 * 1024 - 1024;      // room for the kernel's static LDS
+  return share > needed ? share : needed;
+}
+
 template <int K, int MB, int PRE, bool PREROT> int launch_linear_v(const LinearArgs& a, int grid, size_t lds, hipStream_t st) {
   constexpr int P = K <= 4 ? 4 : (K <= 6 ? 3 : 2);          // wave-steps of weights in flight
   auto kern = k_linear<K, MB, P, (PRE < P ? PRE : P), PREROT>;
+  lds = balanced_lds_request(lds, grid);
   if (lds > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }

@@ -87,22 +87,28 @@ __device__ __forceinline__ void halves32(float v, float& even, float& odd) {
   const u2s r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
   even = __uint_as_float(r.x); odd = __uint_as_float(r.y);
 }
-template <int H> __device__ __forceinline__ void butterfly_dpp(float& a, int lane) {
-  const float p = lane_xor_dpp<H>(a);
-  a = (lane & H) ? (p - a) : (a + p);
+// One butterfly stage between lanes l and l ^ H: the lane with bit H clear gets a + partner, the other partner - a,
+// i.e. a' = partner + s * a with s = +1 / -1 by that lane bit.
+template <int H> __device__ __forceinline__ void butterfly_dpp(float& a, float s) {
+  a = __builtin_fmaf(a, s, lane_xor_dpp<H>(a));
 }
-__device__ __forceinline__ void butterfly16(float& a, int lane) { float e, o; halves16(a, e, o); a = (lane & 16) ? (e - o) : (e + o); }
-__device__ __forceinline__ void butterfly32(float& a, int lane) { float e, o; halves32(a, e, o); a = (lane & 32) ? (e - o) : (e + o); }
+// rows / halves stages: both values of the pair are visible after the swap; a' = even + s * odd
+__device__ __forceinline__ void butterfly16(float& a, float s) { float e, o; halves16(a, e, o); a = __builtin_fmaf(o, s, e); }
+__device__ __forceinline__ void butterfly32(float& a, float s) { float e, o; halves32(a, e, o); a = __builtin_fmaf(o, s, e); }
 
 // 128-point Walsh-Hadamard butterfly network over one wave: lane holds elements `lane` (a) and `lane + 64` (b).
+// For the stages that fetch the partner (xor 1..8) the sign belongs to the lane's own value; for the swap stages
+// (16, 32) both lanes see (even, odd) and the odd-side lane takes the difference.
 __device__ __forceinline__ void fwht128_wave(float& a, float& b, int lane) {
-  float t = a + b; b = a - b; a = t;
-  butterfly_dpp<1>(a, lane); butterfly_dpp<1>(b, lane);
-  butterfly_dpp<2>(a, lane); butterfly_dpp<2>(b, lane);
-  butterfly_dpp<4>(a, lane); butterfly_dpp<4>(b, lane);
-  butterfly_dpp<8>(a, lane); butterfly_dpp<8>(b, lane);
-  butterfly16(a, lane); butterfly16(b, lane);
-  butterfly32(a, lane); butterfly32(b, lane);
+  const float t = a + b; b = a - b; a = t;
+  const float s1 = (lane & 1) ? -1.f : 1.f, s2 = (lane & 2) ? -1.f : 1.f, s4 = (lane & 4) ? -1.f : 1.f;
+  const float s8 = (lane & 8) ? -1.f : 1.f, s16 = (lane & 16) ? -1.f : 1.f, s32 = (lane & 32) ? -1.f : 1.f;
+  butterfly_dpp<1>(a, s1); butterfly_dpp<1>(b, s1);
+  butterfly_dpp<2>(a, s2); butterfly_dpp<2>(b, s2);
+  butterfly_dpp<4>(a, s4); butterfly_dpp<4>(b, s4);
+  butterfly_dpp<8>(a, s8); butterfly_dpp<8>(b, s8);
+  butterfly16(a, s16); butterfly16(b, s16);
+  butterfly32(a, s32); butterfly32(b, s32);
 }
 // all-lanes reductions over the wave, fixed order
 __device__ __forceinline__ float wave_sum(float v) {
@@ -771,7 +777,10 @@ inline bool plan_for_chunk(int m, int n, int M, int chunk, Plan& pl) {
   const int contributors = chunk >= nblk ? 2 : (nblk + chunk - 1) / chunk + 1;
   const double slot_kb = (double)pl.segmax * contributors * 2 * M * 0.5;
   pl.by_counter = slot_kb > 96.0 ? 1 : 0;
-  pl.prerot = (M >= PREROT_MIN_M && prerot_bytes(n, M) <= PREROT_REGION) ? 1 : 0;
+  // pre-rotation also pays for few rows when every wave would otherwise rotate four or more (row, block) pairs in
+  // each of very many workgroups (output heads: 152064x4096 runs 9 % faster with it)
+  const bool redundant = (M * pl.nbl + 7) / 8 >= 4 && pl.wgs >= 3 * NUM_CU;
+  pl.prerot = ((M >= PREROT_MIN_M || redundant) && prerot_bytes(n, M) <= PREROT_REGION) ? 1 : 0;
   return true;
 }
 
@@ -784,7 +793,14 @@ inline bool make_plan(int m, int n, int M, int nsplit, Plan& pl) {
   const int nblk = n / 128, rbs = m / 128;
   const long vtotal = (long)rbs * nblk;
   pl.mb = M <= 8 ? 1 : (M <= 16 ? 2 : 4);
-  if (nsplit > 0) return plan_for_chunk(m, n, M, nsplit, pl);      // explicit chunk length (tuning)
+  if (nsplit > 0) {                                                 // explicit plan (tuning): chunk length in the low
+    const int chunk = nsplit & 0xFFFFF;                             // 20 bits, bit 30 / 29 = force pre-rotation on / off
+    bool ok = chunk > 0 ? plan_for_chunk(m, n, M, chunk, pl) : false;
+    if (ok && (nsplit & (1 << 30)) && prerot_bytes(n, M) <= PREROT_REGION) pl.prerot = 1;
+    if (ok && (nsplit & (1 << 29))) pl.prerot = 0;
+    return ok;
+  }
+  if (vtotal >= (long)64 * NUM_CU && nblk <= 64 && plan_for_chunk(m, n, M, nblk, pl)) return true;
   double best = 1e30;
   bool found = false;
   const int max_chunk = (int)(vtotal < 4096 ? vtotal : 4096);

@@ -8,7 +8,8 @@ import ctypes
 import os
 
 _CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
-LIB_PATH = os.path.join(_CSRC, "libhtr_gfx950.so")
+# HTR_GFX950_LIB names another build of the same library (e.g. a tuning build); it must exist, there is no fallback
+LIB_PATH = os.environ.get("HTR_GFX950_LIB") or os.path.join(_CSRC, "libhtr_gfx950.so")
 
 BF16, F16, F32 = 0, 1, 2
 MAX_BATCH = 32

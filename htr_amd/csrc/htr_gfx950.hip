@@ -134,6 +134,18 @@ __device__ __forceinline__ float wave_max(float v) {
   halves32(v, e, o); return fmaxf(e, o);
 }
 
+typedef uint16_t us2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u3 __attribute__((ext_vector_type(3)));
+template <int CTRL> __device__ __forceinline__ uint32_t dpp_mov_u32(uint32_t v) {
+  return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, false);
+}
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+  v = max(v, dpp_mov_u32<0xB1>(v)); v = max(v, dpp_mov_u32<0x4E>(v));
+  v = max(v, dpp_mov_u32<0x141>(dpp_mov_u32<0x1B>(v))); v = max(v, dpp_mov_u32<0x128>(v));
+  u2s r = __builtin_amdgcn_permlane16_swap(v, v, false, false); v = max(r.x, r.y);
+  r = __builtin_amdgcn_permlane32_swap(v, v, false, false); return max(r.x, r.y);
+}
+
 // ------------------------------------------------------------------------------------------------ stream loads
 // The K dwords of lane `lane` start at dword lane*K of the wave's 64*K-dword step: contiguous across the wave.
 template <int K> struct StreamRegs { uint32_t d[K]; };
@@ -156,6 +168,29 @@ template <int K> __device__ __forceinline__ void load_stream(const uint32_t* __r
   }
 }
 
+// The same K dwords through a buffer descriptor: byte offset `off` from the descriptor's base; out-of-range lanes read
+// zeros without touching memory.  Streaming data: non-temporal.
+template <int K> __device__ __forceinline__ void load_stream_buffer(__amdgpu_buffer_rsrc_t rsrc, int off, StreamRegs<K>& r) {
+  constexpr int NT = 2;
+  if constexpr (K == 2) {
+    u2 v = __builtin_amdgcn_raw_buffer_load_b64(rsrc, off, 0, NT); r.d[0] = v.x; r.d[1] = v.y;
+  } else if constexpr (K == 3) {
+    u3 v = __builtin_amdgcn_raw_buffer_load_b96(rsrc, off, 0, NT); r.d[0] = v.x; r.d[1] = v.y; r.d[2] = v.z;
+  } else if constexpr (K == 4) {
+    u4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, NT); r.d[0] = v.x; r.d[1] = v.y; r.d[2] = v.z; r.d[3] = v.w;
+  } else {
+    u4 v = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, NT); r.d[0] = v.x; r.d[1] = v.y; r.d[2] = v.z; r.d[3] = v.w;
+    if constexpr (K == 5) {
+      r.d[4] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, off + 16, 0, NT);
+    } else if constexpr (K == 6) {
+      u2 t = __builtin_amdgcn_raw_buffer_load_b64(rsrc, off + 16, 0, NT); r.d[4] = t.x; r.d[5] = t.y;
+    } else if constexpr (K == 7) {
+      u3 t = __builtin_amdgcn_raw_buffer_load_b96(rsrc, off + 16, 0, NT); r.d[4] = t.x; r.d[5] = t.y; r.d[6] = t.z;
+    } else {
+      u4 t = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off + 16, 0, NT); r.d[4] = t.x; r.d[5] = t.y; r.d[6] = t.z; r.d[7] = t.w;
+    }
+  }
+}
 // ------------------------------------------------------------------------------------------------ decode core
 // V[0] = the dword before the lane's first dword (history), V[1..K] = the lane's dwords.  Local step u (0..31) is
 // trellis step t = 32q + u; its state is the 16 bits of V that start at bit 16 + (u + 1) * K (bit 0 = MSB of V[0]).
@@ -197,41 +232,40 @@ __device__ __forceinline__ int history_lane_byteaddr(int lane) { return ((lane &
 // The step space of one linear is (128-row block rb, 128-column block blk), row-major: virtual step v = rb * nblk + blk.
 // It is cut into equal contiguous chunks, one per workgroup, so the workgroup count can be a multiple of the CU count
 // whatever the shape.  A chunk may end inside a row block and continue in the next one; each piece of a row block a
-// chunk covers is a "segment" and yields one partial.
-struct LinearArgs {
-  const uint32_t* qw;
+// chunk covers is a "segment" and yields one partial.  The workgroup whose chunk holds the LAST step of a row block
+// finishes that block: it adds the partials of the chunks before it (which can only concern its first segment) to
+// its own and applies the output side.  Every other segment of a chunk is complete by itself; only a chunk's last
+// segment can be a contribution to a later chunk's row block, so one partial slot per workgroup is enough.
+
+// arguments the kernel needs late (epilogue) or only on the pre-rotated path
+struct LinearTail {
   const uint16_t* scales;
-  const uint8_t* su;
   const uint8_t* sv;
-  const void* x;
   const void* bias;
   void* y;
-  uint32_t* cnt;    // [m/128] arrival counters (election by counter only); zero on entry and on exit
-  float* part;      // [workgroups][segmax][2][M][128] partials per segment and tile parity; all-zero on entry and on exit
-  int m, n, M;
-  const _Float16* xt_g;   // pre-rotated activations [M][n] f16 (only when prerot)
+  const _Float16* xt_g;   // pre-rotated activations [M][n] f16 (only when PREROT)
   const float* xs_g;      // their per-(row, block, tile parity) sums [M][n/128][2]
   const float* sc_g;      // per-row activation scale [M]
-  int prerot;             // 1: x~ was produced by k_rotate; 0: this kernel rotates its own column blocks
-  int chunk;        // virtual steps per workgroup
-  int segmax;       // partial slots reserved per workgroup
-  int by_counter;   // 1: elect the finisher of a row block with an arrival counter; 0: by reading every contributor's slot
-  int x_dtype, y_dtype;
+  uint32_t* status;       // workspace word that collects kernel-side failures (bit 0: a finisher gave up waiting)
   float cbscale;
+  int spin_limit;         // polls of the contributors' slots before a finisher gives up
 };
 
-constexpr int MAX_SEG = 64;    // row-block segments one workgroup may produce
-constexpr int PAIR_REGS = 4;   // (activation row, 128-column block) pairs a wave keeps in registers across the barrier
+constexpr int ROT_PAIRS = 16;  // (activation row, 128-column block) pairs a workgroup may rotate by itself
 
-// LDS layout (dynamic): [xt: (M + 1) rows x row_halves f16][pmax: M * nbl f32][xs: M * nbl * 2 f32 (per tile parity)][sc: M f32]
+// LDS layout (dynamic): [xt: (M + 1) rows x row_halves f16][xs: M * nbl * 2 f32 (per tile parity)][sc: M f32]
+//                       [fin: segfin x M x 128 f32, partials of the row blocks this workgroup finishes]
 // nbl = number of distinct column blocks a chunk touches = min(chunk, n / 128)
 // One rotated 128-column block is stored as [columns 0..7 of tiles 0..7][columns 8..15 of tiles 0..7] (2 x 64 halves), and
 // rows are padded by 16 halves: the 16-byte B-operand reads of 8 consecutive lanes (4 activation rows x 2 tile parities)
 // then cover 128 contiguous-mod-128 bytes, i.e. every LDS bank once.
 __host__ __device__ inline int xt_row_halves(int nbl) { return nbl * 128 + 16; }
 __device__ __forceinline__ int xt_slot(int j) { return ((j >> 3) & 1) * 64 + (j >> 4) * 8 + (j & 7); }   // element j of a block
-__host__ __device__ inline size_t lds_bytes(int M, int nbl) {
-  return (size_t)(M + 1) * xt_row_halves(nbl) * 2 + (size_t)M * nbl * 4 * 3 + (size_t)M * 4;
+__host__ __device__ inline size_t lds_fin_offset(int M, int nbl) {
+  return ((size_t)(M + 1) * xt_row_halves(nbl) * 2 + (size_t)M * nbl * 4 * 2 + (size_t)M * 4 + 15) / 16 * 16;
+}
+__host__ __device__ inline size_t lds_bytes(int M, int nbl, int segfin) {
+  return lds_fin_offset(M, nbl) + (size_t)segfin * M * 128 * 4;
 }
 
 // power-of-two activation scale 2^e with sqrt(128) * amax / 2^e in (8192, 16384]: |H128 x| / sqrt(128) <= sqrt(128) * max|x|,
@@ -243,8 +277,8 @@ __device__ __forceinline__ int scale_exponent(float amax) {
 }
 __device__ __forceinline__ float pow2f(int e) { return __uint_as_float((uint32_t)(127 + e) << 23); }
 
-// Rotation of all activation rows ahead of the linear kernel (used from 3 rows up, where every workgroup rotating its
-// own column blocks would repeat the same work hundreds of times): one workgroup per row.
+// Rotation of all activation rows ahead of the linear kernel (used where every workgroup rotating its own column
+// blocks would repeat too much work, and for float32 activations): one workgroup per row.
 __global__ __launch_bounds__(WG_THREADS) void k_rotate(const void* __restrict__ x, const uint8_t* __restrict__ su, int n, int x_dtype,
                                                        _Float16* __restrict__ xt_g, float* __restrict__ xs_g, float* __restrict__ sc_g) {
   __shared__ float s_max[WG_WAVES];
@@ -286,179 +320,179 @@ template <int K> __device__ __forceinline__ void decode_step(const StreamRegs<K>
   d.a[3] = win.template group8<24>();
 }
 
-template <int K, int MB, int P, int PRE, bool PREROT>
-__global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
-  static_assert(PRE <= P, "pre-decoded steps come out of the prefetch registers");
+// Nothing may move across a weight-stream load: the loads of a wave must issue in program order, one per step, so
+// that the number of loads in flight behind any buffer is the same on every path and the wait in front of a decode
+// leaves the other P - 1 loads outstanding.
+#define HTR_PIN() __builtin_amdgcn_sched_barrier(0)
+
+template <int K, int MB, int P, bool PREROT>
+__global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restrict__ qw, const void* __restrict__ x,
+                                                       const uint8_t* __restrict__ su, float* __restrict__ part,
+                                                       int m, int n, int M, int chunk, int flags,
+                                                       const LinearTail t) {
   extern __shared__ __align__(16) unsigned char lds[];
-  __shared__ int s_finish[MAX_SEG];
   const int lane = threadIdx.x & 63;
   const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));   // wave index, provably uniform: keeps the
                                                                            // strip addressing on the scalar unit
-  const int nblk = a.n >> 7, rbs = a.m >> 7;
-  const int M = a.M;
+  const int nblk = n >> 7, rbs = m >> 7;
   const int vtotal = rbs * nblk;
-  const int v0 = blockIdx.x * a.chunk, nsteps = min(vtotal, v0 + a.chunk) - v0;
+  const int v0 = blockIdx.x * chunk, nsteps = min(vtotal, v0 + chunk) - v0;
   const int rb_first = v0 / nblk, c0 = v0 - rb_first * nblk;     // first row block and first column block of the chunk
   const bool all_blocks = nsteps >= nblk;                        // chunk touches every column block
   const int nbl = all_blocks ? nblk : nsteps;                    // distinct column blocks; LDS slot of block b:
-  const int rowh = xt_row_halves(min(a.chunk, nblk));            //   b if all_blocks, else (b - c0) mod nblk
+  const int nblmax = min(chunk, nblk);                           //   b if all_blocks, else (b - c0) mod nblk
+  const int rowh = xt_row_halves(nblmax);
+  const int x_dtype = flags & 3, y_dtype = (flags >> 2) & 3;
 
   _Float16* xt = (_Float16*)lds;
-  float* s_pmax = (float*)(lds + (size_t)(M + 1) * rowh * 2);
-  float* s_xs = s_pmax + M * min(a.chunk, nblk);
-  float* s_sc = s_xs + 2 * M * min(a.chunk, nblk);     // activation scale per row
+  float* s_xs = (float*)(lds + (size_t)(M + 1) * rowh * 2);
+  float* s_sc = s_xs + 2 * M * nblmax;                 // activation scale per row
+  float* s_fin = (float*)(lds + lds_fin_offset(M, nblmax));
 
-  // ---- input rotation of the chunk's column blocks: x~ = f16( H128(su . x) / sqrt(128) / sc ), sc a power of two per
-  // activation row.  Pass 1 loads x (sign applied) and publishes max|x| per (row, block); pass 2 rotates, scales, converts.
   const int npairs = M * nbl;
   auto pair_col = [&](int li) { int b = all_blocks ? li : c0 + li; if (b >= nblk) b -= nblk; return b * 128; };
-  float xa[PAIR_REGS], xb[PAIR_REGS];
-  constexpr bool prerot = PREROT;   // x~ comes from k_rotate instead of being rotated here
   for (int i = threadIdx.x; i < rowh / 2; i += WG_THREADS) ((uint32_t*)(xt + (size_t)M * rowh))[i] = 0u;   // zero row
-  // with pre-rotated activations: 16-byte pieces of this chunk's x~ slice, issued before the weight stream
+
+  // ---- activations first: they head the longest dependency chain.  Every wave loads all (row, block) pairs of the
+  // chunk (a dword = two 16-bit elements per lane and pair) so that it knows max|x| of a row without a barrier; it
+  // rotates pairs w and w + 8.  Register t holds pair (w + 8 (t & 1) + (t >> 1)) mod 16: own pairs sit in 0 and 1.
+  uint32_t xr[ROT_PAIRS];
+  int prow[ROT_PAIRS];                  // activation row of the pair in register t (uniform)
+  uint32_t sb[2] = {0u, 0u};            // su bytes of the own pairs
   constexpr int COPY_REGS = 4;
   u4 cp[COPY_REGS];
   const int ncopy = npairs * 16;                 // 16 pieces of 8 halves per (row, block) pair
-  if constexpr (prerot) {
+  if constexpr (!PREROT) {
+    // descriptors over x and su: a pair beyond the chunk's last one gets an out-of-range offset and reads zeros, so
+    // all loads issue back to back without branches
+    const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)x, 0, M * n * 2, 0x00020000);
+    const __amdgpu_buffer_rsrc_t srsrc = __builtin_amdgcn_make_buffer_rsrc((void*)su, 0, n >> 3, 0x00020000);
+    constexpr int OUT_OF_RANGE = 0x7FFFFF00;
+    // (row, block) of the pairs walked by the even and the odd registers: they start at pairs w and w + 8 and advance
+    // by one pair, wrapping from pair 15 to pair 0
+    int mr[2], li[2], pi[2];
+    pi[0] = w; pi[1] = w + 8;
+    mr[0] = w / nbl; li[0] = w - mr[0] * nbl;
+    mr[1] = (w + 8) / nbl; li[1] = w + 8 - mr[1] * nbl;
 #pragma unroll
-    for (int t = 0; t < COPY_REGS; ++t) {
-      const int ci = threadIdx.x + t * WG_THREADS;
+    for (int tt = 0; tt < ROT_PAIRS; ++tt) {
+      const int h = tt & 1;
+      const bool live = pi[h] < npairs;
+      const int col = pair_col(li[h]);
+      prow[tt] = live ? mr[h] : -1;
+      xr[tt] = __builtin_amdgcn_raw_buffer_load_b32(xrsrc, live ? (mr[h] * n + col) * 2 + 4 * lane : OUT_OF_RANGE, 0, 0);
+      if (tt < 2) sb[tt] = (uint32_t)(uint8_t)__builtin_amdgcn_raw_buffer_load_b8(srsrc, live ? (col >> 3) + (lane >> 2) : OUT_OF_RANGE, 0, 0);
+      if (++pi[h] == ROT_PAIRS) { pi[h] = 0; mr[h] = 0; li[h] = 0; }
+      else if (++li[h] == nbl) { li[h] = 0; ++mr[h]; }
+    }
+  } else {
+    // with pre-rotated activations: 16-byte pieces of this chunk's x~ slice
+#pragma unroll
+    for (int tt = 0; tt < COPY_REGS; ++tt) {
+      const int ci = threadIdx.x + tt * WG_THREADS;
       if (ci < ncopy) {
         const int pi = ci >> 4, mrow = pi / nbl, li = pi - mrow * nbl;
-        cp[t] = *(const u4*)(a.xt_g + (size_t)mrow * a.n + pair_col(li) + (ci & 15) * 8);
+        cp[tt] = *(const u4*)(t.xt_g + (size_t)mrow * n + pair_col(li) + (ci & 15) * 8);
       }
     }
   }
-#pragma unroll
-  for (int t = 0; t < PAIR_REGS; ++t) {     // x first: loads return in order, and x heads the longest dependency chain
-    const int pi = w + t * WG_WAVES;
-    xa[t] = 0.f; xb[t] = 0.f;
-    if (!prerot && pi < npairs) {
-      const int mrow = pi / nbl, li = pi - mrow * nbl, col = pair_col(li);
-      const size_t base = (size_t)mrow * a.n + col;
-      xa[t] = load_elem(a.x, a.x_dtype, base + lane) * sign_of(a.su, col + lane);
-      xb[t] = load_elem(a.x, a.x_dtype, base + lane + 64) * sign_of(a.su, col + lane + 64);
-    }
-  }
 
-  // ---- start the weight stream.  This wave's strip of row block rb is tile row rb * 8 + w; its 8 tiles of column
-  // block blk are 64 * K contiguous dwords; a strip is contiguous over blk, the same strip of the next row block
-  // starts 8 strips later.
-  constexpr int STEP_DWORDS = 64 * K;
-  const size_t strip_dwords = (size_t)nblk * STEP_DWORDS;
-  const uint32_t* pf_ptr = a.qw + (size_t)(rb_first * 8 + w) * strip_dwords + (size_t)c0 * STEP_DWORDS;   // uniform
-  const int lane_dwords = lane * K;
+  // ---- the weight stream.  This wave's strip of row block rb is tile row rb * 8 + w; its 8 tiles of column block blk
+  // are 64 * K contiguous dwords; a strip is contiguous over blk, the same strip of the next row block starts 8 strips
+  // later.  The stream is addressed through a buffer descriptor that covers exactly the wave's bytes of this chunk:
+  // a load beyond the last step is out of range, returns zeros and costs no memory traffic, so every step can issue
+  // its load unconditionally.
+  constexpr int STEP_BYTES = 256 * K;
+  const uint32_t strip_bytes = (uint32_t)nblk * STEP_BYTES;
+  const uint32_t* wave_base = qw + ((size_t)(rb_first * 8 + w) * nblk + (size_t)c0) * (STEP_BYTES / 4);   // uniform
+  const int last_wraps = (c0 + nsteps - 1) / nblk;
+  const uint32_t extent = (uint32_t)nsteps * STEP_BYTES + (uint32_t)last_wraps * 7u * strip_bytes;
+  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)wave_base, 0, (int)extent, 0x00020000);
+  int pf_off = lane * 4 * K;         // byte offset of this lane's dwords in the next step to load
   int pf_blk = c0;
   StreamRegs<K> buf[P];
   auto prefetch = [&](StreamRegs<K>& dst) {
-    load_stream<K>(pf_ptr + lane_dwords, dst);
-    pf_ptr += STEP_DWORDS;
-    if (++pf_blk == nblk) { pf_blk = 0; pf_ptr += 7 * strip_dwords; }
+    HTR_PIN();
+    load_stream_buffer<K>(rsrc, pf_off, dst);
+    pf_off += STEP_BYTES;
+    if (++pf_blk == nblk) { pf_blk = 0; pf_off += 7 * (int)strip_bytes; }
+    HTR_PIN();
   };
-  const bool rotator = !prerot && w < npairs;      // this wave rotates at least one pair
-  if constexpr (prerot) {
 #pragma unroll
-    for (int p = 0; p < P; ++p)
-      if (p < nsteps) prefetch(buf[p]);
-  }
-  if constexpr (!prerot) {
-#pragma unroll
-  for (int t = 0; t < PAIR_REGS; ++t) {
-    const int pi = w + t * WG_WAVES;
-    if (pi < npairs) {
-      const float mx = wave_max(fmaxf(fabsf(xa[t]), fabsf(xb[t])));
-      if (lane == 0) s_pmax[pi] = mx;
-    }
-  }
-  // The weight stream starts only now, after x has arrived: when every wave of the chip bursts its first weight loads
-  // at once, an x load issued just before them takes about twice as long, and x heads the critical chain, while the
-  // rotation below hides the weight latency anyway.
-  asm volatile("" ::: "memory");
-#pragma unroll
-  for (int p = 0; p < P; ++p)
-    if (p < nsteps) prefetch(buf[p]);
-  for (int pi = w + PAIR_REGS * WG_WAVES; pi < npairs; pi += WG_WAVES) {   // more pairs than registers: max only, reload later
-    const int mrow = pi / nbl, li = pi - mrow * nbl;
-    const size_t base = (size_t)mrow * a.n + pair_col(li);
-    const float mx = wave_max(fmaxf(fabsf(load_elem(a.x, a.x_dtype, base + lane)), fabsf(load_elem(a.x, a.x_dtype, base + lane + 64))));
-    if (lane == 0) s_pmax[pi] = mx;
-  }
-  __syncthreads();
-  // max|x| of activation row mrow over the chunk's blocks: lanes read the per-block maxima, one wave reduction
-  auto row_amax = [&](int mrow) {
-    float v = 0.f;
-    for (int k = lane; k < nbl; k += 64) v = fmaxf(v, s_pmax[mrow * nbl + k]);
-    return wave_max(v);
-  };
-  auto rotate_pair = [&](int pi, float va, float vb) {
-    const int mrow = pi / nbl, li = pi - mrow * nbl;
-    const int e = scale_exponent(row_amax(mrow));
-    const float inv_sc = pow2f(-e);
-    if (li == 0 && lane == 0) s_sc[mrow] = pow2f(e);
-    va *= inv_sc; vb *= inv_sc;
-    fwht128_wave(va, vb, lane);
-    const _Float16 ha = (_Float16)(va * INV_SQRT128), hb = (_Float16)(vb * INV_SQRT128);
-    xt[(size_t)mrow * rowh + li * 128 + xt_slot(lane)] = ha;
-    xt[(size_t)mrow * rowh + li * 128 + xt_slot(lane + 64)] = hb;
-    // sum of the rounded x~ per tile parity (element j sits in tile j / 16; lane and lane + 64 share the parity)
-    float se, so;
-    wave_sum_by_row_parity((float)ha + (float)hb, se, so);
-    if (lane == 0) { s_xs[2 * pi] = se; s_xs[2 * pi + 1] = so; }
-  };
-  // The rotation is a long chain of dependent instructions that every wave of the workgroup waits for: run it at
-  // raised priority so that decoding waves on the same SIMD do not starve it.
-  __builtin_amdgcn_s_setprio(3);
-#pragma unroll
-  for (int t = 0; t < PAIR_REGS; ++t) {   // unrolled: the chains of a wave's pairs interleave
-    const int pi = w + t * WG_WAVES;
-    if (pi < npairs) rotate_pair(pi, xa[t], xb[t]);
-  }
-  for (int pi = w + PAIR_REGS * WG_WAVES; pi < npairs; pi += WG_WAVES) {
-    const int mrow = pi / nbl, li = pi - mrow * nbl, col = pair_col(li);
-    const size_t base = (size_t)mrow * a.n + col;
-    rotate_pair(pi, load_elem(a.x, a.x_dtype, base + lane) * sign_of(a.su, col + lane),
-                load_elem(a.x, a.x_dtype, base + lane + 64) * sign_of(a.su, col + lane + 64));
-  }
-  __builtin_amdgcn_s_setprio(0);
+  for (int p = 0; p < P; ++p) prefetch(buf[p]);
 
+  if constexpr (!PREROT) {
+    // max|x| per row over the chunk's blocks, for the rows of the two own pairs: 16-bit float patterns order like
+    // their magnitudes once the sign bit is cleared, so the maximum is taken on the raw bits, two elements at a time
+    const bool is_bf16 = x_dtype == HTR_BF16;
+    us2 mx0 = {0, 0}, mx1 = {0, 0};
+#pragma unroll
+    for (int tt = 0; tt < ROT_PAIRS; ++tt) {
+      const uint32_t mag = xr[tt] & 0x7FFF7FFFu;          // pairs beyond npairs hold zeros
+      const uint32_t k0 = prow[tt] == prow[0] ? 0xFFFFFFFFu : 0u, k1 = prow[tt] == prow[1] ? 0xFFFFFFFFu : 0u;
+      mx0 = __builtin_elementwise_max(mx0, __builtin_bit_cast(us2, mag & k0));
+      mx1 = __builtin_elementwise_max(mx1, __builtin_bit_cast(us2, mag & k1));
+    }
+    auto row_scale_exp = [&](us2 mx) {
+      uint32_t v = max((uint32_t)mx.x, (uint32_t)mx.y);
+      v = wave_max_u32(v);
+      const float amax = is_bf16 ? __uint_as_float(v << 16) : f16_bits_to_float((uint16_t)v);
+      return scale_exponent(amax);
+    };
+    auto rotate_pair = [&](int pi, uint32_t raw, uint32_t sbyte, us2 mx) {
+      const int mrow = pi / nbl, li = pi - mrow * nbl;
+      const int e = row_scale_exp(mx);
+      const float inv_sc = pow2f(-e);
+      if (li == 0 && lane == 0) s_sc[mrow] = pow2f(e);
+      uint32_t lo, hi;
+      if (is_bf16) { lo = raw << 16; hi = raw & 0xFFFF0000u; }
+      else { lo = __float_as_uint(f16_bits_to_float((uint16_t)raw)); hi = __float_as_uint(f16_bits_to_float((uint16_t)(raw >> 16))); }
+      const int sh = 2 * (lane & 3);                                 // bits of elements 2 lane, 2 lane + 1 in the su byte
+      lo ^= ((sbyte >> sh) & 1u) << 31;
+      hi ^= ((sbyte >> (sh + 1)) & 1u) << 31;
+      float va = __uint_as_float(lo) * inv_sc, vb = __uint_as_float(hi) * inv_sc;
+      // lane holds elements 2 lane and 2 lane + 1: the in-lane stage is index bit 0, lane bit i is index bit i + 1
+      fwht128_wave(va, vb, lane);
+      const _Float16 ha = (_Float16)(va * INV_SQRT128), hb = (_Float16)(vb * INV_SQRT128);
+      const uint32_t packed = (uint32_t)__builtin_bit_cast(uint16_t, ha) | ((uint32_t)__builtin_bit_cast(uint16_t, hb) << 16);
+      *(uint32_t*)(xt + (size_t)mrow * rowh + li * 128 + xt_slot(2 * lane)) = packed;
+      // sum of the rounded x~ per tile parity: element 2 lane sits in tile lane / 8, so the parity is lane bit 3
+      float s = (float)ha + (float)hb;
+      s += lane_xor_dpp<1>(s); s += lane_xor_dpp<2>(s); s += lane_xor_dpp<4>(s);
+      float e0, o0;
+      halves16(s, e0, o0); s = e0 + o0;
+      halves32(s, e0, o0); s = e0 + o0;
+      if ((lane & ~8) == 0) s_xs[2 * pi + (lane >> 3)] = s;
+    };
+    if (w < npairs) rotate_pair(w, xr[0], sb[0], mx0);
+    if (w + 8 < npairs) rotate_pair(w + 8, xr[1], sb[1], mx1);
   } else {
     // copy the slice into LDS; sums per (row, block, parity) come with it
 #pragma unroll
-    for (int t = 0; t < COPY_REGS; ++t) {
-      const int ci = threadIdx.x + t * WG_THREADS;
+    for (int tt = 0; tt < COPY_REGS; ++tt) {
+      const int ci = threadIdx.x + tt * WG_THREADS;
       if (ci < ncopy) {
         const int pi = ci >> 4, mrow = pi / nbl, li = pi - mrow * nbl;
-        *(u4*)(xt + (size_t)mrow * rowh + li * 128 + (ci & 1) * 64 + ((ci & 15) >> 1) * 8) = cp[t];
+        *(u4*)(xt + (size_t)mrow * rowh + li * 128 + (ci & 1) * 64 + ((ci & 15) >> 1) * 8) = cp[tt];
       }
     }
     for (int ci = threadIdx.x + COPY_REGS * WG_THREADS; ci < ncopy; ci += WG_THREADS) {
       const int pi = ci >> 4, mrow = pi / nbl, li = pi - mrow * nbl;
       *(u4*)(xt + (size_t)mrow * rowh + li * 128 + (ci & 1) * 64 + ((ci & 15) >> 1) * 8) =
-          *(const u4*)(a.xt_g + (size_t)mrow * a.n + pair_col(li) + (ci & 15) * 8);
+          *(const u4*)(t.xt_g + (size_t)mrow * n + pair_col(li) + (ci & 15) * 8);
     }
     for (int i = threadIdx.x; i < npairs * 2; i += WG_THREADS) {
       const int pi = i >> 1, mrow = pi / nbl, li = pi - mrow * nbl;
-      s_xs[i] = a.xs_g[((size_t)mrow * nblk + (pair_col(li) >> 7)) * 2 + (i & 1)];
+      s_xs[i] = t.xs_g[((size_t)mrow * nblk + (pair_col(li) >> 7)) * 2 + (i & 1)];
     }
   }
-  // ---- decode the first steps into registers.  Waves that rotate nothing do it before the x~ barrier, while the
-  // rotating waves sit in their dependency chains, so the rotation latency is not dead time; rotating waves go to
-  // the barrier at once and decode the same steps after it.
+
+  // ---- decode step 0 while the other waves finish their rotations, then meet
   const int hist = history_lane_byteaddr(lane);
-  DecodedStep<K> pre[PRE];
-  auto predecode = [&]() {
-#pragma unroll
-    for (int p = 0; p < PRE; ++p)
-      if (p < nsteps) {
-        decode_step<K>(buf[p], hist, pre[p]);
-        if (p + P < nsteps) prefetch(buf[p]);
-      }
-  };
-  // (when most waves rotate, the few that do not would only delay the barrier by decoding first)
-  const bool early = !rotator && npairs <= WG_WAVES / 2;
-  if (early) predecode();
+  DecodedStep<K> cur;
+  decode_step<K>(buf[0], hist, cur);
+  prefetch(buf[0]);
   __syncthreads();
-  if (!early) predecode();
 
   // ---- per-lane constants of the product and of the partial store
   // MFMA operands: row i = lane % 16 = (tile parity h = i / 8, row pair q = i % 8); B column c = lane % 16 carries
@@ -481,18 +515,17 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
     xsoff[mb] = live ? 2 * (mrow * nbl) + par : -1;
     offs[mb] = 0.f; sc[mb] = 0.f;
     if (live) {
-      if constexpr (prerot) sc[mb] = a.sc_g[mrow];
+      if constexpr (PREROT) sc[mb] = t.sc_g[mrow];
       else sc[mb] = s_sc[mrow];
     }
   }
-  const size_t slot_floats = (size_t)2 * M * 128;          // one segment: [parity][M][128]
-  float* myslot = a.part + (size_t)blockIdx.x * a.segmax * slot_floats + 16 * w + 8 * (g & 1);
 
   f4 acc[MB][2];
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) { acc[mb][0] = f4{0.f, 0.f, 0.f, 0.f}; acc[mb][1] = f4{0.f, 0.f, 0.f, 0.f}; }
 
   int cur_blk = c0, cur_li = all_blocks ? c0 : 0, cur_seg = 0, done = 0;
+  // product of the decoded step with the chunk's rotated activations, and the end of a segment
   auto consume = [&](const DecodedStep<K>& d) {
     h8 B0[MB], B1[MB];
 #pragma unroll
@@ -505,124 +538,119 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const LinearArgs a) {
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) acc[mb][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[0], B0[mb], acc[mb][0], 0, 0, 0);
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) acc[mb][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[1], B1[mb], acc[mb][0], 0, 0, 0);
-#pragma unroll
     for (int mb = 0; mb < MB; ++mb) acc[mb][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[2], B0[mb], acc[mb][1], 0, 0, 0);
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) acc[mb][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[1], B1[mb], acc[mb][0], 0, 0, 0);
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) acc[mb][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[3], B1[mb], acc[mb][1], 0, 0, 0);
     ++done; ++cur_blk; ++cur_li;
     const bool row_end = cur_blk == nblk;
     if (row_end || done == nsteps) {
-      // end of a segment: this wave's strip partials, one per tile parity, with the 1534 offset removed and the
-      // activation scale undone.  Stored with the lowest mantissa bit set (never the all-zero pattern), device scope
-      // (written through), not waited for here.
-      float* dst0 = myslot + (size_t)cur_seg * slot_floats;
+      // End of a segment: this wave's strip partial per activation row, the 1534 offset removed, the activation scale
+      // undone, the two tile parities added (the parity-1 lane of a value is lane ^ 33).  A segment that ends its
+      // row block is finished by this workgroup and goes to LDS; a chunk that ends inside a row block leaves its
+      // last partial in the workgroup's slot, stored with the lowest mantissa bit set (never the all-zero pattern),
+      // device scope (written through), not waited for.
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
         const int mrow = mb * 8 + (n16 >> 1);
-        if (xsoff[mb] >= 0) {
-          uint32_t* dst = (uint32_t*)(dst0 + (size_t)(par * M + mrow) * 128);
+        float tot[8];
 #pragma unroll
-          for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < 4; ++j)
 #pragma unroll
-            for (int rr = 0; rr < 2; ++rr)
-              __hip_atomic_store(dst + 2 * j + rr, __float_as_uint((acc[mb][rr][j] - offs[mb]) * sc[mb]) | 1u,
-                                 __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          for (int rr = 0; rr < 2; ++rr) {
+            const float v = xsoff[mb] >= 0 ? (acc[mb][rr][j] - offs[mb]) * sc[mb] : 0.f;
+            float lo_half, hi_half;
+            halves32(lane_xor_dpp<1>(v), lo_half, hi_half);
+            tot[2 * j + rr] = v + hi_half;            // meaningful in lanes < 32 with an even column
+          }
+        if (lane < 32 && (n16 & 1) == 0 && mrow < M) {
+          const int rowi = 16 * w + 8 * (g & 1);
+          if (row_end) {
+            float* dst = s_fin + ((size_t)cur_seg * M + mrow) * 128 + rowi;
+            *(f4*)dst = f4{tot[0], tot[1], tot[2], tot[3]};
+            *(f4*)(dst + 4) = f4{tot[4], tot[5], tot[6], tot[7]};
+          } else {
+            uint32_t* dst = (uint32_t*)(part + ((size_t)blockIdx.x * M + mrow) * 128 + rowi);
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+              __hip_atomic_store(dst + i, __float_as_uint(tot[i]) | 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
         }
         acc[mb][0] = f4{0.f, 0.f, 0.f, 0.f}; acc[mb][1] = f4{0.f, 0.f, 0.f, 0.f};
         offs[mb] = 0.f;
       }
-      ++cur_seg;
-      if (row_end) { cur_blk = 0; if (all_blocks) cur_li = 0; }
+      if (row_end) { ++cur_seg; cur_blk = 0; if (all_blocks) cur_li = 0; }
     }
   };
 
-#pragma unroll
-  for (int p = 0; p < PRE; ++p)
-    if (p < nsteps) consume(pre[p]);
-
-  // ---- main loop: one 128-column block (8 tiles of this wave's strip) per step; buffer p holds step v with v % P == p
-  for (int vb = PRE; vb < nsteps; vb += P) {
+  // ---- main loop: one 128-column block (8 tiles of this wave's strip) per step.  Step v multiplies what the previous
+  // step decoded, then decodes step v + 1 out of buffer (v + 1) % P while the matrix unit works, then refills it.
+  for (int vb = 0; vb < nsteps; vb += P) {
 #pragma unroll
     for (int pp = 0; pp < P; ++pp) {
-      constexpr int dummy = 0; (void)dummy;
-      const int p = (PRE + pp) % P;
       const int v = vb + pp;
+      constexpr int dummy = 0; (void)dummy;
+      StreamRegs<K>& nxt = buf[(pp + 1) % P];
       if (v < nsteps) {
-        DecodedStep<K> d;
-        decode_step<K>(buf[p], hist, d);
-        if (v + P < nsteps) prefetch(buf[p]);
-        consume(d);
+        consume(cur);
+        if (v + 1 < nsteps) decode_step<K>(nxt, hist, cur);
       }
+      prefetch(nxt);
     }
   }
 
-  // ---- cross-workgroup reduction.  The workspace is all-zero between calls.  Device-scope stores are acknowledged
-  // once written through, so after the wait and the barrier every partial of this workgroup is visible device-wide
-  // (a cache-wide writeback would also do, at many times the cost).
-  //   election by slots:   for each row block it touched the workgroup reads the slots of every contributing chunk;
-  //                        if none is zero all have arrived and it finishes the row block.  Several workgroups may
-  //                        see a complete set; they compute bit-identical results (fixed summation order) and store
-  //                        the same values.
-  //   election by counter: one arrival per workgroup and row block; the last one finishes.  Same-address atomics
-  //                        serialise, so this is used only where re-reading the slots would cost more.
-  // Either way the finisher zeroes what it consumed.
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  // ---- output side of the row blocks that end in this chunk (cur_seg of them)
   __syncthreads();
-  const int nseg = cur_seg;
-  if (a.by_counter) {
-    if ((int)threadIdx.x < nseg) {
-      const int rb = rb_first + threadIdx.x;
-      const int j0 = (rb * nblk) / a.chunk, j1 = (rb * nblk + nblk - 1) / a.chunk;
-      s_finish[threadIdx.x] = __hip_atomic_fetch_add(&a.cnt[rb], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (uint32_t)(j1 - j0);
-    }
-    __syncthreads();
-    if ((int)threadIdx.x < nseg && s_finish[threadIdx.x])
-      __hip_atomic_store(&a.cnt[rb_first + threadIdx.x], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-
-  for (int idx = w; idx < nseg * M; idx += WG_WAVES) {
+  const int nfin = cur_seg;
+  const size_t slot_floats = (size_t)M * 128;
+  for (int idx = w; idx < nfin * M; idx += WG_WAVES) {
     const int seg = idx / M, mrow = idx - seg * M, rb = rb_first + seg;
-    if (a.by_counter && !s_finish[seg]) continue;
     const int r0 = rb * 128 + lane, r1 = r0 + 64;
-    const float rs0 = f16_bits_to_float(a.scales[r0]) * a.cbscale, rs1 = f16_bits_to_float(a.scales[r1]) * a.cbscale;
-    const float sg0 = sign_of(a.sv, r0), sg1 = sign_of(a.sv, r1);
+    const float rs0 = f16_bits_to_float(t.scales[r0]) * t.cbscale, rs1 = f16_bits_to_float(t.scales[r1]) * t.cbscale;
+    const float sg0 = sign_of(t.sv, r0), sg1 = sign_of(t.sv, r1);
     float b0v = 0.f, b1v = 0.f;
-    if (a.bias != nullptr) { b0v = load_elem(a.bias, a.y_dtype, r0); b1v = load_elem(a.bias, a.y_dtype, r1); }
-    // contributors: chunks j0..j1 overlap row block rb; chunk j holds it in its segment rb - (first row block of j)
-    const int j0 = (rb * nblk) / a.chunk, j1 = (rb * nblk + nblk - 1) / a.chunk;
-    const int sj0 = rb - (j0 * a.chunk) / nblk;              // every later contributor starts inside rb: segment 0
+    if (t.bias != nullptr) { b0v = load_elem(t.bias, y_dtype, r0); b1v = load_elem(t.bias, y_dtype, r1); }
     float v0s = 0.f, v1s = 0.f;
-    bool missing = false;
-    auto slot_of = [&](int j) {
-      return (uint32_t*)(a.part + ((size_t)j * a.segmax + (j == j0 ? sj0 : 0)) * slot_floats + (size_t)mrow * 128);
-    };
-#pragma unroll 8
-    for (int j = j0; j <= j1; ++j) {
-      const uint32_t* pp = slot_of(j);
-#pragma unroll
-      for (int pr = 0; pr < 2; ++pr) {
-        const uint32_t u0 = __hip_atomic_load(pp + (size_t)pr * M * 128 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const uint32_t u1 = __hip_atomic_load(pp + (size_t)pr * M * 128 + lane + 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        missing |= (u0 == 0u) | (u1 == 0u);
-        v0s += __uint_as_float(u0); v1s += __uint_as_float(u1);
+    bool failed = false;
+    if (seg == 0 && c0 != 0) {
+      // earlier chunks hold the beginning of this row block: chunks j0 .. blockIdx.x - 1, each in its own slot.  They
+      // were dispatched before this workgroup, so waiting for them cannot deadlock; the wait is bounded all the same.
+      const int j0 = (rb * nblk) / chunk, j1 = (int)blockIdx.x;
+      int tries = 0;
+      for (;;) {
+        bool missing = false;
+        v0s = 0.f; v1s = 0.f;
+        for (int j = j0; j < j1; ++j) {
+          const uint32_t* pp = (const uint32_t*)(part + (size_t)j * slot_floats + (size_t)mrow * 128);
+          const uint32_t u0 = __hip_atomic_load(pp + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          const uint32_t u1 = __hip_atomic_load(pp + lane + 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          missing |= (u0 == 0u) | (u1 == 0u);
+          v0s += __uint_as_float(u0); v1s += __uint_as_float(u1);
+        }
+        if (!__any(missing)) break;
+        if (++tries >= t.spin_limit) { failed = true; break; }
+        __builtin_amdgcn_s_sleep(2);
+      }
+      if (!failed) {
+        for (int j = j0; j < j1; ++j) {          // leave the workspace zero for the next call
+          uint32_t* pp = (uint32_t*)(part + (size_t)j * slot_floats + (size_t)mrow * 128);
+          __hip_atomic_store(pp + lane, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(pp + lane + 64, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      } else if (lane == 0) {
+        __hip_atomic_fetch_or(t.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
-    if (__any(missing)) continue;             // some contributor has not arrived yet: a later workgroup finishes this row
-    for (int j = j0; j <= j1; ++j) {          // leave the workspace zero for the next call
-      uint32_t* pp = slot_of(j);
-#pragma unroll
-      for (int pr = 0; pr < 2; ++pr) {
-        __hip_atomic_store(pp + (size_t)pr * M * 128 + lane, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __hip_atomic_store(pp + (size_t)pr * M * 128 + lane + 64, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
-    }
+    const float* own = s_fin + ((size_t)seg * M + mrow) * 128;
+    v0s += own[lane]; v1s += own[lane + 64];
     v0s *= rs0; v1s *= rs1;
     fwht128_wave(v0s, v1s, lane);
     v0s = v0s * INV_SQRT128 * sg0 + b0v;
     v1s = v1s * INV_SQRT128 * sg1 + b1v;
-    store_elem(a.y, a.y_dtype, (size_t)mrow * a.m + r0, v0s);
-    store_elem(a.y, a.y_dtype, (size_t)mrow * a.m + r1, v1s);
+    if (failed) { v0s = __builtin_nanf(""); v1s = v0s; }
+    store_elem(t.y, y_dtype, (size_t)mrow * m + r0, v0s);
+    store_elem(t.y, y_dtype, (size_t)mrow * m + r1, v1s);
   }
 }
 
@@ -748,73 +776,68 @@ __global__ __launch_bounds__(512) void k_dequant_w(const uint32_t* __restrict__ 
 
 // ------------------------------------------------------------------------------------------------ host side
 thread_local int g_last_hip_error = 0;
+int g_spin_limit = 1 << 20;     // polls (about a microsecond each) before a finishing workgroup gives up
 
-struct Plan { int chunk, wgs, segmax, nbl, mb, by_counter, prerot; size_t lds; };
+struct Plan { int chunk, wgs, segfin, nbl, mb, prerot; size_t lds; };
 
-constexpr int PREROT_MIN_M = 6;   // from this many rows on the activations are rotated once by k_rotate
-// The pre-rotated activations live in a fixed region between the counters and the partial slots: partial slots must be
-// all-zero between calls, and no call may leave other data where a later call of another shape expects such slots.
+// Workspace: [256-byte header: status word][pre-rotated activations, fixed region][one partial slot per workgroup].
+// Partial slots must be all-zero between calls, and no call may leave other data where a later call of another shape
+// expects such slots: hence the fixed region in front of them.
+constexpr size_t WS_HEADER = 256;
 constexpr size_t PREROT_REGION = (size_t)4 << 20;
 inline size_t align256(size_t v) { return (v + 255) / 256 * 256; }
 // bytes of the pre-rotated activations, their block sums and the row scales
 inline size_t prerot_bytes(int n, int M) { return align256((size_t)M * n * 2) + align256((size_t)M * (n / 128) * 8) + align256((size_t)M * 4); }
 
 constexpr int NUM_CU = 256;
-constexpr int MAX_ROW_BLOCKS = 16384;                       // counter region: one word per 128-row block
-inline size_t counters_bytes() { return (size_t)MAX_ROW_BLOCKS * 4; }
+constexpr int MAX_ROW_BLOCKS = 16384;
+constexpr int MAX_CHUNK = 4096;
 
 inline bool plan_for_chunk(int m, int n, int M, int chunk, Plan& pl) {
   const int nblk = n / 128, rbs = m / 128;
   const long vtotal = (long)rbs * nblk;
-  if (chunk < 1 || chunk > vtotal) return false;
+  if (chunk < 1 || chunk > vtotal || chunk > MAX_CHUNK) return false;
   pl.chunk = chunk;
   pl.wgs = (int)((vtotal + chunk - 1) / chunk);
-  pl.segmax = chunk == 1 ? 1 : (chunk + nblk - 2) / nblk + 1;
+  pl.segfin = (chunk + nblk - 1) / nblk;            // row blocks that can end inside one chunk
   pl.nbl = chunk < nblk ? chunk : nblk;
-  pl.lds = lds_bytes(M, pl.nbl);
-  if (pl.segmax > MAX_SEG || pl.lds > (size_t)LDS_BUDGET) return false;
-  // bytes a workgroup re-reads when finishers are elected by slots: per segment, every contributor's two parities
-  const int contributors = chunk >= nblk ? 2 : (nblk + chunk - 1) / chunk + 1;
-  const double slot_kb = (double)pl.segmax * contributors * 2 * M * 0.5;
-  pl.by_counter = slot_kb > 96.0 ? 1 : 0;
-  // pre-rotation also pays for few rows when every wave would otherwise rotate four or more (row, block) pairs in
-  // each of very many workgroups (output heads: 152064x4096 runs 9 % faster with it)
-  const bool redundant = (M * pl.nbl + 7) / 8 >= 4 && pl.wgs >= 3 * NUM_CU;
-  pl.prerot = ((M >= PREROT_MIN_M || redundant) && prerot_bytes(n, M) <= PREROT_REGION) ? 1 : 0;
+  pl.lds = lds_bytes(M, pl.nbl, pl.segfin);
+  if (pl.lds > (size_t)LDS_BUDGET) return false;
+  // a workgroup rotates its own column blocks while that is at most ROT_PAIRS (row, block) pairs; beyond that the
+  // activations are rotated once, ahead of the launch
+  pl.prerot = M * pl.nbl > ROT_PAIRS ? 1 : 0;
+  if (pl.prerot && prerot_bytes(n, M) > PREROT_REGION) return false;
   return true;
 }
 
 // Picks the chunk length (virtual steps per workgroup) with a cost model in microseconds fitted to chunk-length sweeps
-// on MI355X (K4, batch 1): a fixed latency chain of ~6 us (launch, x fetch, rotation, store acknowledgement, slot reads,
-// output rotation); ~0.8 us per step while every CU holds at most one workgroup, 0.7 us per step and resident
-// workgroup beyond that, plus contention when workgroups share a CU; chunks that do not divide a row of column blocks
-// (or are not whole rows) cost ~35 % more; every extra contributor to a row block adds slot reads.
+// on MI355X (K4): a fixed latency chain (launch, x fetch, rotation, partial exchange, output rotation), a per-step cost
+// that grows with the workgroups resident per CU, a penalty for chunks that do not tile the rows of column blocks,
+// the extra launch of a pre-rotation, and the slot reads of a finisher per contributor.
 inline bool make_plan(int m, int n, int M, int nsplit, Plan& pl) {
   const int nblk = n / 128, rbs = m / 128;
   const long vtotal = (long)rbs * nblk;
   pl.mb = M <= 8 ? 1 : (M <= 16 ? 2 : 4);
   if (nsplit > 0) {                                                 // explicit plan (tuning): chunk length in the low
-    const int chunk = nsplit & 0xFFFFF;                             // 20 bits, bit 30 / 29 = force pre-rotation on / off
+    const int chunk = nsplit & 0xFFFFF;                             // 20 bits, bit 30 = force pre-rotation
     bool ok = chunk > 0 ? plan_for_chunk(m, n, M, chunk, pl) : false;
-    if (ok && (nsplit & (1 << 30)) && prerot_bytes(n, M) <= PREROT_REGION) pl.prerot = 1;
-    if (ok && (nsplit & (1 << 29))) pl.prerot = 0;
+    if (ok && (nsplit & (1 << 30))) { if (prerot_bytes(n, M) <= PREROT_REGION) pl.prerot = 1; else ok = false; }
     return ok;
   }
   if (vtotal >= (long)64 * NUM_CU && nblk <= 64 && plan_for_chunk(m, n, M, nblk, pl)) return true;
   double best = 1e30;
   bool found = false;
-  const int max_chunk = (int)(vtotal < 4096 ? vtotal : 4096);
+  const int max_chunk = (int)(vtotal < MAX_CHUNK ? vtotal : MAX_CHUNK);
   for (int chunk = 1; chunk <= max_chunk; ++chunk) {
     Plan c;
     c.mb = pl.mb;
     if (!plan_for_chunk(m, n, M, chunk, c)) continue;
     const double k = (double)c.wgs / NUM_CU;
-    const double step = (k <= 1.0 ? 0.8 : 0.7 * k) * (1.0 + 0.25 * (pl.mb - 1));
+    const double waves = k <= 1.0 ? 1.0 : (double)((c.wgs + NUM_CU - 1) / NUM_CU);     // workgroups on the fullest CU
+    const double step = (waves <= 1.0 ? 0.55 : 0.42 * waves) * (1.0 + 0.25 * (pl.mb - 1));
     const bool aligned = (nblk % chunk == 0) || (chunk % nblk == 0);
-    const int pairs_per_wave = c.prerot ? 1 : (M * c.nbl + 7) / 8;
     const int contributors = chunk >= nblk ? 1 : (nblk + chunk - 1) / chunk;
-    const double t = 6.0 + (k > 1.0 ? 1.5 : 0.0) + 0.15 * (pairs_per_wave - 1) + step * chunk * (aligned ? 1.0 : 1.35)
-                     + 0.1 * contributors + (c.by_counter ? 0.4 * contributors + 1.0 : 0.0);
+    const double t = 4.5 + (c.prerot ? 2.5 : 0.0) + step * chunk * (aligned ? 1.0 : 1.15) + 0.05 * contributors;
     if (t < best) { best = t; pl = c; found = true; }
   }
   return found;
@@ -827,35 +850,38 @@ constexpr size_t CU_LDS_BYTES = 160 * 1024;
 inline size_t balanced_lds_request(size_t needed, int grid) {
   const int k = (grid + NUM_CU - 1) / NUM_CU;
   if (k > 4) return needed;
-  const size_t share = (CU_LDS_BYTES / k) / 1024 * 1024 - 1024;      // room for the kernel's static LDS
+  const size_t share = (CU_LDS_BYTES / k) / 1024 * 1024 - 1024;
   return share > needed ? share : needed;
 }
 
-template <int K, int MB, int PRE, bool PREROT> int launch_linear_v(const LinearArgs& a, int grid, size_t lds, hipStream_t st) {
+struct LinearLaunch {
+  const uint32_t* qw; const void* x; const uint8_t* su; float* part;
+  int m, n, M, chunk, flags;
+  LinearTail tail;
+};
+
+template <int K, int MB, bool PREROT> int launch_linear_v(const LinearLaunch& a, int grid, size_t lds, hipStream_t st) {
   constexpr int P = K <= 4 ? 4 : (K <= 6 ? 3 : 2);          // wave-steps of weights in flight
-  auto kern = k_linear<K, MB, P, (PRE < P ? PRE : P), PREROT>;
+  auto kern = k_linear<K, MB, P, PREROT>;
   lds = balanced_lds_request(lds, grid);
   if (lds > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
   }
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(WG_THREADS), lds, st, a);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(WG_THREADS), lds, st, a.qw, a.x, a.su, a.part, a.m, a.n, a.M, a.chunk, a.flags, a.tail);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
   return HTR_OK;
 }
-// Steps decoded ahead of the x~ barrier: deep (more registers, fewer resident waves) only for short chunks, where the
-// prologue latency is a large part of the kernel; long chunks prefer occupancy.
-template <int K, bool PREROT> int launch_linear_kr(const LinearArgs& a, int mb, int grid, size_t lds, hipStream_t st) {
-  const bool deep = a.chunk <= 8;
+template <int K, bool PREROT> int launch_linear_kr(const LinearLaunch& a, int mb, int grid, size_t lds, hipStream_t st) {
   switch (mb) {
-    case 1: return deep ? launch_linear_v<K, 1, 4, PREROT>(a, grid, lds, st) : launch_linear_v<K, 1, 1, PREROT>(a, grid, lds, st);
-    case 2: return deep ? launch_linear_v<K, 2, 2, PREROT>(a, grid, lds, st) : launch_linear_v<K, 2, 1, PREROT>(a, grid, lds, st);
-    default: return launch_linear_v<K, 4, 1, PREROT>(a, grid, lds, st);
+    case 1: return launch_linear_v<K, 1, PREROT>(a, grid, lds, st);
+    case 2: return launch_linear_v<K, 2, PREROT>(a, grid, lds, st);
+    default: return launch_linear_v<K, 4, PREROT>(a, grid, lds, st);
   }
 }
-template <int K> int launch_linear_k(const LinearArgs& a, int mb, int grid, size_t lds, hipStream_t st) {
-  return a.prerot ? launch_linear_kr<K, true>(a, mb, grid, lds, st) : launch_linear_kr<K, false>(a, mb, grid, lds, st);
+template <int K> int launch_linear_k(const LinearLaunch& a, bool prerot, int mb, int grid, size_t lds, hipStream_t st) {
+  return prerot ? launch_linear_kr<K, true>(a, mb, grid, lds, st) : launch_linear_kr<K, false>(a, mb, grid, lds, st);
 }
 
 #define HTR_FOR_K(K, EXPR)                 \
@@ -902,7 +928,7 @@ size_t htr_workspace_bytes(int m, int n, int K, int M, int nsplit) {
   if (K < 2 || K > 8 || m <= 0 || n <= 0 || m % 128 || n % 128 || m / 128 > MAX_ROW_BLOCKS || M < 1 || M > HTR_MAX_BATCH) return 0;
   Plan pl;
   if (!make_plan(m, n, M, nsplit, pl)) return 0;
-  return counters_bytes() + PREROT_REGION + (size_t)pl.wgs * pl.segmax * 2 * M * 128 * sizeof(float);
+  return WS_HEADER + PREROT_REGION + (size_t)pl.wgs * M * 128 * sizeof(float);
 }
 
 int htr_linear_plan(int m, int n, int K, int M, int nsplit, int* out6) {
@@ -912,9 +938,11 @@ int htr_linear_plan(int m, int n, int K, int M, int nsplit, int* out6) {
   if (M < 1 || M > HTR_MAX_BATCH) return HTR_ERR_BATCH;
   Plan pl;
   if (!make_plan(m, n, M, nsplit, pl)) return HTR_ERR_SPLIT;
-  out6[0] = pl.chunk; out6[1] = pl.wgs; out6[2] = pl.segmax; out6[3] = pl.nbl; out6[4] = pl.by_counter; out6[5] = (int)pl.lds;
+  out6[0] = pl.chunk; out6[1] = pl.wgs; out6[2] = pl.segfin; out6[3] = pl.nbl; out6[4] = pl.prerot; out6[5] = (int)pl.lds;
   return HTR_OK;
 }
+
+void htr_set_spin_limit(int polls) { g_spin_limit = polls < 1 ? 1 : polls; }
 
 int htr_linear(const void* qweight, const void* scales, const void* su, const void* sv, const void* x, const void* bias,
                void* y, int m, int n, int K, int M, int x_dtype, int y_dtype, int nsplit, void* workspace,
@@ -929,33 +957,35 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
     return HTR_ERR_ALIGN;
   Plan pl;
   if (!make_plan(m, n, M, nsplit, pl)) return HTR_ERR_SPLIT;
+  // the in-kernel rotation reads 16-bit elements in pairs: float32 activations, and rows that do not start on a
+  // 4-byte boundary, take the pre-rotation
+  const bool prerot = pl.prerot || x_dtype == HTR_F32 || ((uintptr_t)x & 3);
+  if (prerot && prerot_bytes(n, M) > PREROT_REGION) return HTR_ERR_SPLIT;
   const size_t need = htr_workspace_bytes(m, n, K, M, nsplit);
   if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255)) return HTR_ERR_WORKSPACE;
 
-  LinearArgs a;
-  a.qw = (const uint32_t*)qweight; a.scales = (const uint16_t*)scales; a.su = (const uint8_t*)su; a.sv = (const uint8_t*)sv;
-  a.x = x; a.bias = bias; a.y = y;
-  a.cnt = (uint32_t*)workspace;
-  unsigned char* wsp = (unsigned char*)workspace + counters_bytes();
-  a.prerot = pl.prerot; a.xt_g = nullptr; a.xs_g = nullptr; a.sc_g = nullptr;
-  if (pl.prerot) {
-    a.xt_g = (const _Float16*)wsp;
-    a.xs_g = (const float*)(wsp + align256((size_t)M * n * 2));
-    a.sc_g = (const float*)(wsp + align256((size_t)M * n * 2) + align256((size_t)M * (n / 128) * 8));
-  }
+  unsigned char* wsp = (unsigned char*)workspace + WS_HEADER;
+  LinearLaunch a;
+  a.qw = (const uint32_t*)qweight; a.x = x; a.su = (const uint8_t*)su;
   a.part = (float*)(wsp + PREROT_REGION);
-  a.m = m; a.n = n; a.M = M; a.chunk = pl.chunk; a.segmax = pl.segmax; a.by_counter = pl.by_counter;
-  a.x_dtype = x_dtype; a.y_dtype = y_dtype;
-  a.cbscale = htr_cbscale();
-  const int grid = pl.wgs;
+  a.m = m; a.n = n; a.M = M; a.chunk = pl.chunk; a.flags = x_dtype | (y_dtype << 2);
+  LinearTail& t = a.tail;
+  t.scales = (const uint16_t*)scales; t.sv = (const uint8_t*)sv; t.bias = bias; t.y = y;
+  t.xt_g = nullptr; t.xs_g = nullptr; t.sc_g = nullptr;
+  t.status = (uint32_t*)workspace;
+  t.cbscale = htr_cbscale();
+  t.spin_limit = g_spin_limit;
   hipStream_t st = (hipStream_t)stream;
-  if (pl.prerot) {
-    hipLaunchKernelGGL(k_rotate, dim3(M), dim3(WG_THREADS), 0, st, x, (const uint8_t*)su, n, x_dtype, (_Float16*)a.xt_g,
-                       (float*)a.xs_g, (float*)a.sc_g);
+  if (prerot) {
+    t.xt_g = (const _Float16*)wsp;
+    t.xs_g = (const float*)(wsp + align256((size_t)M * n * 2));
+    t.sc_g = (const float*)(wsp + align256((size_t)M * n * 2) + align256((size_t)M * (n / 128) * 8));
+    hipLaunchKernelGGL(k_rotate, dim3(M), dim3(WG_THREADS), 0, st, x, (const uint8_t*)su, n, x_dtype, (_Float16*)t.xt_g,
+                       (float*)t.xs_g, (float*)t.sc_g);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
   }
-  HTR_FOR_K(K, return launch_linear_k<KK>(a, pl.mb, grid, pl.lds, st));
+  HTR_FOR_K(K, return launch_linear_k<KK>(a, prerot, pl.mb, pl.wgs, pl.lds, st));
   return HTR_OK;
 }
 

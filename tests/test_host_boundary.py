@@ -68,13 +68,14 @@ def test_validation_codes_without_gpu(L):
 def test_launch_plan_is_consistent(L, m, n, M):
     out = (ctypes.c_int * 6)()
     assert L.htr_linear_plan(m, n, 4, M, 0, out) == 0
-    chunk, wgs, segmax, nbl, by_counter, lds = list(out)
+    chunk, wgs, segfin, nbl, prerot, lds = list(out)
     nblk, rbs = n // 128, m // 128
     assert chunk >= 1 and (wgs - 1) * chunk < rbs * nblk <= wgs * chunk          # chunks tile the step space exactly
     assert nbl == min(chunk, nblk) and lds <= 64 * 1024
-    assert segmax >= 1 and (chunk <= 1 or segmax >= (chunk + nblk - 2) // nblk + 1)
+    assert segfin == (chunk + nblk - 1) // nblk                                  # row blocks that can end inside one chunk
+    assert prerot == (1 if M * nbl > 16 else 0)                                  # a workgroup rotates at most 16 pairs itself
     need = L.htr_workspace_bytes(m, n, 4, M, 0)
-    assert need >= 65536 + wgs * segmax * 2 * M * 128 * 4
+    assert need >= 256 + wgs * M * 128 * 4                                       # header + one partial slot per workgroup
     # an explicit chunk length is honoured
     assert L.htr_linear_plan(m, n, 4, M, 1, out) == 0 or M * 128 * 2 > 60000
     if out[0] == 1:

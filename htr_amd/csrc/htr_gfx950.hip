@@ -90,7 +90,9 @@ __device__ __forceinline__ void halves32(float v, float& even, float& odd) {
 // One butterfly stage between lanes l and l ^ H: the lane with bit H clear gets a + partner, the other partner - a,
 // i.e. a' = partner + s * a with s = +1 / -1 by that lane bit.
 template <int H> __device__ __forceinline__ void butterfly_dpp(float& a, float s) {
-  a = __builtin_fmaf(a, s, lane_xor_dpp<H>(a));
+  // own value with the sign of s, added to the partner's: an xor and an add whose DPP operand fetches the partner
+  const float own = __uint_as_float(__float_as_uint(a) ^ (__float_as_uint(s) & 0x80000000u));
+  a = lane_xor_dpp<H>(a) + own;
 }
 // rows / halves stages: both values of the pair are visible after the swap; a' = even + s * odd
 __device__ __forceinline__ void butterfly16(float& a, float s) { float e, o; halves16(a, e, o); a = __builtin_fmaf(o, s, e); }
@@ -197,6 +199,17 @@ template <int K> __device__ __forceinline__ void load_stream_buffer(__amdgpu_buf
 template <int K> struct Window {
   uint32_t V[K + 1];
   uint32_t mid[K];     // mid[w] = bits [32w + 16, 32w + 48) of V, for windows that straddle two dwords
+  // the same in two parts: everything that does not involve the history dword, then the rest
+  __device__ __forceinline__ void build_tail(const StreamRegs<K>& r) {
+#pragma unroll
+    for (int k = 0; k < K; ++k) V[k + 1] = r.d[k];
+#pragma unroll
+    for (int k = 1; k < K; ++k) mid[k] = __builtin_amdgcn_alignbit(V[k], V[k + 1], 16);
+  }
+  __device__ __forceinline__ void build_head(uint32_t prev) {
+    V[0] = prev;
+    mid[0] = __builtin_amdgcn_alignbit(V[0], V[1], 16);
+  }
   __device__ __forceinline__ void build(const StreamRegs<K>& r, uint32_t prev) {
     V[0] = prev;
 #pragma unroll
@@ -247,13 +260,14 @@ struct LinearTail {
   const float* xs_g;      // their per-(row, block, tile parity) sums [M][n/128][2]
   const float* sc_g;      // per-row activation scale [M]
   uint32_t* status;       // workspace word that collects kernel-side failures (bit 0: a finisher gave up waiting)
+  unsigned long long chunk_magic;   // ceil(2^40 / chunk): step index -> chunk index
   float cbscale;
   int spin_limit;         // polls of the contributors' slots before a finisher gives up
 };
 
 constexpr int ROT_PAIRS = 16;  // (activation row, 128-column block) pairs a workgroup may rotate by itself
 
-// LDS layout (dynamic): [xt: (M + 1) rows x row_halves f16][xs: M * nbl * 2 f32 (per tile parity)][sc: M f32]
+// LDS layout (dynamic): [xt: (M + 1) rows x row_halves f16][xs: M * nbl * 2 f32 (per tile parity)][sc: M f32][pmax: 16 f32]
 //                       [fin: segfin x M x 128 f32, partials of the row blocks this workgroup finishes]
 // nbl = number of distinct column blocks a chunk touches = min(chunk, n / 128)
 // One rotated 128-column block is stored as [columns 0..7 of tiles 0..7][columns 8..15 of tiles 0..7] (2 x 64 halves), and
@@ -262,7 +276,7 @@ constexpr int ROT_PAIRS = 16;  // (activation row, 128-column block) pairs a wor
 __host__ __device__ inline int xt_row_halves(int nbl) { return nbl * 128 + 16; }
 __device__ __forceinline__ int xt_slot(int j) { return ((j >> 3) & 1) * 64 + (j >> 4) * 8 + (j & 7); }   // element j of a block
 __host__ __device__ inline size_t lds_fin_offset(int M, int nbl) {
-  return ((size_t)(M + 1) * xt_row_halves(nbl) * 2 + (size_t)M * nbl * 4 * 2 + (size_t)M * 4 + 15) / 16 * 16;
+  return ((size_t)(M + 1) * xt_row_halves(nbl) * 2 + (size_t)M * nbl * 4 * 2 + (size_t)M * 4 + ROT_PAIRS * 4 + 15) / 16 * 16;
 }
 __host__ __device__ inline size_t lds_bytes(int M, int nbl, int segfin) {
   return lds_fin_offset(M, nbl) + (size_t)segfin * M * 128 * 4;
@@ -312,12 +326,18 @@ __global__ __launch_bounds__(WG_THREADS) void k_rotate(const void* __restrict__ 
 template <int K> struct DecodedStep { h8 a[4]; };   // MFMA A operands of one step: (row 2q | 2q+1) x (columns 0..7 | 8..15)
 
 template <int K> __device__ __forceinline__ void decode_step(const StreamRegs<K>& r, int hist, DecodedStep<K>& d) {
+  // The history dword travels through the LDS crossbar.  Only the first states of the lane reach into it, so their
+  // group is decoded last, behind a scheduling fence: the crossbar latency hides behind the other three groups.
+  const uint32_t prev = (uint32_t)__builtin_amdgcn_ds_bpermute(hist, (int)r.d[K - 1]);
+  __builtin_amdgcn_sched_barrier(0);
   Window<K> win;
-  win.build(r, (uint32_t)__builtin_amdgcn_ds_bpermute(hist, (int)r.d[K - 1]));
-  d.a[0] = win.template group8<0>();
+  win.build_tail(r);
   d.a[1] = win.template group8<8>();
   d.a[2] = win.template group8<16>();
   d.a[3] = win.template group8<24>();
+  __builtin_amdgcn_sched_barrier(0);
+  win.build_head(prev);
+  d.a[0] = win.template group8<0>();
 }
 
 // Nothing may move across a weight-stream load: the loads of a wave must issue in program order, one per step, so
@@ -329,15 +349,19 @@ template <int K, int MB, int P, bool PREROT>
 __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restrict__ qw, const void* __restrict__ x,
                                                        const uint8_t* __restrict__ su, float* __restrict__ part,
                                                        int m, int n, int M, int chunk, int flags,
-                                                       const LinearTail t) {
+                                                       unsigned long long nblk_magic, const LinearTail t) {
   extern __shared__ __align__(16) unsigned char lds[];
   const int lane = threadIdx.x & 63;
   const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));   // wave index, provably uniform: keeps the
                                                                            // strip addressing on the scalar unit
-  const int nblk = n >> 7, rbs = m >> 7;
-  const int vtotal = rbs * nblk;
+  const int nblk = n >> 7;
+  const int vtotal = (m >> 7) * nblk;
   const int v0 = blockIdx.x * chunk, nsteps = min(vtotal, v0 + chunk) - v0;
-  const int rb_first = v0 / nblk, c0 = v0 - rb_first * nblk;     // first row block and first column block of the chunk
+  // v / nblk for v < 2^24 by multiplication: nblk_magic = ceil(2^40 / nblk)
+  auto div_nblk = [&](int v) { return (int)(((unsigned long long)(unsigned)v * nblk_magic) >> 40); };
+  const int rb_first = div_nblk(v0), c0 = v0 - rb_first * nblk;  // first row block and first column block of the chunk
+  const int last_wraps = div_nblk(c0 + nsteps - 1);              // row-block changes before the chunk's last step
+  const int nfin = div_nblk(c0 + nsteps);                        // row blocks that end inside the chunk
   const bool all_blocks = nsteps >= nblk;                        // chunk touches every column block
   const int nbl = all_blocks ? nblk : nsteps;                    // distinct column blocks; LDS slot of block b:
   const int nblmax = min(chunk, nblk);                           //   b if all_blocks, else (b - c0) mod nblk
@@ -347,43 +371,35 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
   _Float16* xt = (_Float16*)lds;
   float* s_xs = (float*)(lds + (size_t)(M + 1) * rowh * 2);
   float* s_sc = s_xs + 2 * M * nblmax;                 // activation scale per row
+  float* s_pmax = s_sc + M;                            // max|x| per (row, block) pair
   float* s_fin = (float*)(lds + lds_fin_offset(M, nblmax));
 
   const int npairs = M * nbl;
   auto pair_col = [&](int li) { int b = all_blocks ? li : c0 + li; if (b >= nblk) b -= nblk; return b * 128; };
-  for (int i = threadIdx.x; i < rowh / 2; i += WG_THREADS) ((uint32_t*)(xt + (size_t)M * rowh))[i] = 0u;   // zero row
 
-  // ---- activations first: they head the longest dependency chain.  Every wave loads all (row, block) pairs of the
-  // chunk (a dword = two 16-bit elements per lane and pair) so that it knows max|x| of a row without a barrier; it
-  // rotates pairs w and w + 8.  Register t holds pair (w + 8 (t & 1) + (t >> 1)) mod 16: own pairs sit in 0 and 1.
-  uint32_t xr[ROT_PAIRS];
-  int prow[ROT_PAIRS];                  // activation row of the pair in register t (uniform)
-  uint32_t sb[2] = {0u, 0u};            // su bytes of the own pairs
+  // ---- activations first: they head the longest dependency chain.  Wave w rotates the (row, block) pairs w and w + 8:
+  // one dword (two 16-bit elements) per lane and pair, plus the su byte that holds the two sign bits.  Descriptors
+  // over x and su: a pair beyond the chunk's last one gets an out-of-range offset and reads zeros, so the loads
+  // issue back to back without branches.
+  constexpr int NPW = ROT_PAIRS / WG_WAVES;   // pairs per wave
+  uint32_t xr[NPW], sb[NPW];
+  int prow[NPW], pli[NPW];
   constexpr int COPY_REGS = 4;
   u4 cp[COPY_REGS];
   const int ncopy = npairs * 16;                 // 16 pieces of 8 halves per (row, block) pair
   if constexpr (!PREROT) {
-    // descriptors over x and su: a pair beyond the chunk's last one gets an out-of-range offset and reads zeros, so
-    // all loads issue back to back without branches
     const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)x, 0, M * n * 2, 0x00020000);
     const __amdgpu_buffer_rsrc_t srsrc = __builtin_amdgcn_make_buffer_rsrc((void*)su, 0, n >> 3, 0x00020000);
     constexpr int OUT_OF_RANGE = 0x7FFFFF00;
-    // (row, block) of the pairs walked by the even and the odd registers: they start at pairs w and w + 8 and advance
-    // by one pair, wrapping from pair 15 to pair 0
-    int mr[2], li[2], pi[2];
-    pi[0] = w; pi[1] = w + 8;
-    mr[0] = w / nbl; li[0] = w - mr[0] * nbl;
-    mr[1] = (w + 8) / nbl; li[1] = w + 8 - mr[1] * nbl;
 #pragma unroll
-    for (int tt = 0; tt < ROT_PAIRS; ++tt) {
-      const int h = tt & 1;
-      const bool live = pi[h] < npairs;
-      const int col = pair_col(li[h]);
-      prow[tt] = live ? mr[h] : -1;
-      xr[tt] = __builtin_amdgcn_raw_buffer_load_b32(xrsrc, live ? (mr[h] * n + col) * 2 + 4 * lane : OUT_OF_RANGE, 0, 0);
-      if (tt < 2) sb[tt] = (uint32_t)(uint8_t)__builtin_amdgcn_raw_buffer_load_b8(srsrc, live ? (col >> 3) + (lane >> 2) : OUT_OF_RANGE, 0, 0);
-      if (++pi[h] == ROT_PAIRS) { pi[h] = 0; mr[h] = 0; li[h] = 0; }
-      else if (++li[h] == nbl) { li[h] = 0; ++mr[h]; }
+    for (int tt = 0; tt < NPW; ++tt) {
+      const int pi = w + tt * WG_WAVES;
+      const bool live = pi < npairs;
+      prow[tt] = M == 1 ? 0 : pi / nbl;
+      pli[tt] = pi - prow[tt] * nbl;
+      const int col = pair_col(pli[tt]);
+      xr[tt] = __builtin_amdgcn_raw_buffer_load_b32(xrsrc, live ? (prow[tt] * n + col) * 2 + 4 * lane : OUT_OF_RANGE, 0, 0);
+      sb[tt] = (uint32_t)(uint8_t)__builtin_amdgcn_raw_buffer_load_b8(srsrc, live ? (col >> 3) + (lane >> 2) : OUT_OF_RANGE, 0, 0);
     }
   } else {
     // with pre-rotated activations: 16-byte pieces of this chunk's x~ slice
@@ -405,7 +421,6 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
   constexpr int STEP_BYTES = 256 * K;
   const uint32_t strip_bytes = (uint32_t)nblk * STEP_BYTES;
   const uint32_t* wave_base = qw + ((size_t)(rb_first * 8 + w) * nblk + (size_t)c0) * (STEP_BYTES / 4);   // uniform
-  const int last_wraps = (c0 + nsteps - 1) / nblk;
   const uint32_t extent = (uint32_t)nsteps * STEP_BYTES + (uint32_t)last_wraps * 7u * strip_bytes;
   const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)wave_base, 0, (int)extent, 0x00020000);
   int pf_off = lane * 4 * K;         // byte offset of this lane's dwords in the next step to load
@@ -421,51 +436,62 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
 #pragma unroll
   for (int p = 0; p < P; ++p) prefetch(buf[p]);
 
+  for (int i = threadIdx.x; i < rowh / 2; i += WG_THREADS) ((uint32_t*)(xt + (size_t)M * rowh))[i] = 0u;   // zero row
+
+  // ---- rotation, first half: unpack, apply su, publish max|x| of the pair, rotate unscaled in float32 (H128 is
+  // linear and the scale is a power of two, so scaling afterwards gives the same bits)
+  float ra[NPW], rb[NPW];
   if constexpr (!PREROT) {
-    // max|x| per row over the chunk's blocks, for the rows of the two own pairs: 16-bit float patterns order like
-    // their magnitudes once the sign bit is cleared, so the maximum is taken on the raw bits, two elements at a time
     const bool is_bf16 = x_dtype == HTR_BF16;
-    us2 mx0 = {0, 0}, mx1 = {0, 0};
 #pragma unroll
-    for (int tt = 0; tt < ROT_PAIRS; ++tt) {
-      const uint32_t mag = xr[tt] & 0x7FFF7FFFu;          // pairs beyond npairs hold zeros
-      const uint32_t k0 = prow[tt] == prow[0] ? 0xFFFFFFFFu : 0u, k1 = prow[tt] == prow[1] ? 0xFFFFFFFFu : 0u;
-      mx0 = __builtin_elementwise_max(mx0, __builtin_bit_cast(us2, mag & k0));
-      mx1 = __builtin_elementwise_max(mx1, __builtin_bit_cast(us2, mag & k1));
-    }
-    auto row_scale_exp = [&](us2 mx) {
-      uint32_t v = max((uint32_t)mx.x, (uint32_t)mx.y);
-      v = wave_max_u32(v);
-      const float amax = is_bf16 ? __uint_as_float(v << 16) : f16_bits_to_float((uint16_t)v);
-      return scale_exponent(amax);
-    };
-    auto rotate_pair = [&](int pi, uint32_t raw, uint32_t sbyte, us2 mx) {
-      const int mrow = pi / nbl, li = pi - mrow * nbl;
-      const int e = row_scale_exp(mx);
-      const float inv_sc = pow2f(-e);
-      if (li == 0 && lane == 0) s_sc[mrow] = pow2f(e);
+    for (int tt = 0; tt < NPW; ++tt) {
+      const int pi = w + tt * WG_WAVES;
       uint32_t lo, hi;
-      if (is_bf16) { lo = raw << 16; hi = raw & 0xFFFF0000u; }
-      else { lo = __float_as_uint(f16_bits_to_float((uint16_t)raw)); hi = __float_as_uint(f16_bits_to_float((uint16_t)(raw >> 16))); }
+      if (is_bf16) { lo = xr[tt] << 16; hi = xr[tt] & 0xFFFF0000u; }
+      else { lo = __float_as_uint(f16_bits_to_float((uint16_t)xr[tt])); hi = __float_as_uint(f16_bits_to_float((uint16_t)(xr[tt] >> 16))); }
       const int sh = 2 * (lane & 3);                                 // bits of elements 2 lane, 2 lane + 1 in the su byte
-      lo ^= ((sbyte >> sh) & 1u) << 31;
-      hi ^= ((sbyte >> (sh + 1)) & 1u) << 31;
-      float va = __uint_as_float(lo) * inv_sc, vb = __uint_as_float(hi) * inv_sc;
-      // lane holds elements 2 lane and 2 lane + 1: the in-lane stage is index bit 0, lane bit i is index bit i + 1
-      fwht128_wave(va, vb, lane);
-      const _Float16 ha = (_Float16)(va * INV_SQRT128), hb = (_Float16)(vb * INV_SQRT128);
-      const uint32_t packed = (uint32_t)__builtin_bit_cast(uint16_t, ha) | ((uint32_t)__builtin_bit_cast(uint16_t, hb) << 16);
-      *(uint32_t*)(xt + (size_t)mrow * rowh + li * 128 + xt_slot(2 * lane)) = packed;
-      // sum of the rounded x~ per tile parity: element 2 lane sits in tile lane / 8, so the parity is lane bit 3
-      float s = (float)ha + (float)hb;
-      s += lane_xor_dpp<1>(s); s += lane_xor_dpp<2>(s); s += lane_xor_dpp<4>(s);
-      float e0, o0;
-      halves16(s, e0, o0); s = e0 + o0;
-      halves32(s, e0, o0); s = e0 + o0;
-      if ((lane & ~8) == 0) s_xs[2 * pi + (lane >> 3)] = s;
-    };
-    if (w < npairs) rotate_pair(w, xr[0], sb[0], mx0);
-    if (w + 8 < npairs) rotate_pair(w + 8, xr[1], sb[1], mx1);
+      lo ^= ((sb[tt] >> sh) & 1u) << 31;
+      hi ^= ((sb[tt] >> (sh + 1)) & 1u) << 31;
+      ra[tt] = __uint_as_float(lo); rb[tt] = __uint_as_float(hi);
+      if (pi < npairs) {                                             // uniform
+        const float mx = wave_max(fmaxf(fabsf(ra[tt]), fabsf(rb[tt])));
+        if (lane == 0) s_pmax[pi] = mx;
+        // lane holds elements 2 lane and 2 lane + 1: the in-lane stage is index bit 0, lane bit i is index bit i + 1
+        fwht128_wave(ra[tt], rb[tt], lane);
+      }
+    }
+  }
+
+  // ---- decode the first two steps into registers around the activation exchange: they need no x~, and they fill
+  // the time the other waves take to reach the barriers
+  const int hist = history_lane_byteaddr(lane);
+  DecodedStep<K> pre0, cur;
+  decode_step<K>(buf[0], hist, pre0);
+  prefetch(buf[0]);
+
+  if constexpr (!PREROT) {
+    __syncthreads();
+    // rotation, second half: the row's scale from the published maxima, then scale, round to f16, store
+#pragma unroll
+    for (int tt = 0; tt < NPW; ++tt) {
+      const int pi = w + tt * WG_WAVES;
+      if (pi < npairs) {
+        const float amax = wave_max(s_pmax[prow[tt] * nbl + min(lane, nbl - 1)]);
+        const int e = scale_exponent(amax);
+        const float f = pow2f(-e) * INV_SQRT128;
+        if (pli[tt] == 0 && lane == 0) s_sc[prow[tt]] = pow2f(e);
+        const _Float16 ha = (_Float16)(ra[tt] * f), hb = (_Float16)(rb[tt] * f);
+        const uint32_t packed = (uint32_t)__builtin_bit_cast(uint16_t, ha) | ((uint32_t)__builtin_bit_cast(uint16_t, hb) << 16);
+        *(uint32_t*)(xt + (size_t)prow[tt] * rowh + pli[tt] * 128 + xt_slot(2 * lane)) = packed;
+        // sum of the rounded x~ per tile parity: element 2 lane sits in tile lane / 8, so the parity is lane bit 3
+        float s = (float)ha + (float)hb;
+        s += lane_xor_dpp<1>(s); s += lane_xor_dpp<2>(s); s += lane_xor_dpp<4>(s);
+        float e0, o0;
+        halves16(s, e0, o0); s = e0 + o0;
+        halves32(s, e0, o0); s = e0 + o0;
+        if ((lane & ~8) == 0) s_xs[2 * pi + (lane >> 3)] = s;
+      }
+    }
   } else {
     // copy the slice into LDS; sums per (row, block, parity) come with it
 #pragma unroll
@@ -486,12 +512,8 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
       s_xs[i] = t.xs_g[((size_t)mrow * nblk + (pair_col(li) >> 7)) * 2 + (i & 1)];
     }
   }
-
-  // ---- decode step 0 while the other waves finish their rotations, then meet
-  const int hist = history_lane_byteaddr(lane);
-  DecodedStep<K> cur;
-  decode_step<K>(buf[0], hist, cur);
-  prefetch(buf[0]);
+  if (nsteps > 1) decode_step<K>(buf[1 % P], hist, cur);
+  prefetch(buf[1 % P]);
   __syncthreads();
 
   // ---- per-lane constants of the product and of the partial store
@@ -525,16 +547,25 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
   for (int mb = 0; mb < MB; ++mb) { acc[mb][0] = f4{0.f, 0.f, 0.f, 0.f}; acc[mb][1] = f4{0.f, 0.f, 0.f, 0.f}; }
 
   int cur_blk = c0, cur_li = all_blocks ? c0 : 0, cur_seg = 0, done = 0;
-  // product of the decoded step with the chunk's rotated activations, and the end of a segment
-  auto consume = [&](const DecodedStep<K>& d) {
-    h8 B0[MB], B1[MB];
+  // B operands and x~ sums of the step about to be multiplied: read from LDS one step ahead, right after the
+  // previous step's matrix instructions issue, so that their latency hides behind the decode
+  h8 B0[MB], B1[MB];
+  float xsv[MB];
+  float k1534[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) k1534[mb] = xsoff[mb] >= 0 ? 1534.f : 0.f;
+  auto load_b = [&](int li) {
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
-      const _Float16* bp = xt + boff[mb] + cur_li * 128;
+      const _Float16* bp = xt + boff[mb] + li * 128;
       B0[mb] = *(const h8*)bp;
       B1[mb] = *(const h8*)(bp + 64);
-      if (xsoff[mb] >= 0) offs[mb] += 1534.f * s_xs[xsoff[mb] + 2 * cur_li];
+      xsv[mb] = s_xs[max(xsoff[mb], 0) + 2 * li];
     }
+  };
+  load_b(cur_li);
+  // product of the decoded step with the chunk's rotated activations, and the end of a segment
+  auto consume = [&](const DecodedStep<K>& d, bool maybe_last) {
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) acc[mb][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[0], B0[mb], acc[mb][0], 0, 0, 0);
 #pragma unroll
@@ -543,9 +574,14 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
     for (int mb = 0; mb < MB; ++mb) acc[mb][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[1], B1[mb], acc[mb][0], 0, 0, 0);
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) acc[mb][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[3], B1[mb], acc[mb][1], 0, 0, 0);
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) offs[mb] = __builtin_fmaf(k1534[mb], xsv[mb], offs[mb]);
     ++done; ++cur_blk; ++cur_li;
     const bool row_end = cur_blk == nblk;
-    if (row_end || done == nsteps) {
+    const bool seg_end = row_end || (maybe_last && done == nsteps);
+    if (row_end) { cur_blk = 0; if (all_blocks) cur_li = 0; }
+    if (!(maybe_last && done == nsteps)) load_b(cur_li);          // next step's operands (the slot exists: not the last step)
+    if (seg_end) {
       // End of a segment: this wave's strip partial per activation row, the 1534 offset removed, the activation scale
       // undone, the two tile parities added (the parity-1 lane of a value is lane ^ 33).  A segment that ends its
       // row block is finished by this workgroup and goes to LDS; a chunk that ends inside a row block leaves its
@@ -580,53 +616,80 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
         acc[mb][0] = f4{0.f, 0.f, 0.f, 0.f}; acc[mb][1] = f4{0.f, 0.f, 0.f, 0.f};
         offs[mb] = 0.f;
       }
-      if (row_end) { ++cur_seg; cur_blk = 0; if (all_blocks) cur_li = 0; }
+      if (row_end) ++cur_seg;
     }
   };
 
   // ---- main loop: one 128-column block (8 tiles of this wave's strip) per step.  Step v multiplies what the previous
   // step decoded, then decodes step v + 1 out of buffer (v + 1) % P while the matrix unit works, then refills it.
-  for (int vb = 0; vb < nsteps; vb += P) {
+  // Groups of P steps that all have a successor run without bounds checks; the last steps are checked one by one.
+  consume(pre0, true);
+  int v = 1;
+  for (; v + P < nsteps; v += P) {
 #pragma unroll
     for (int pp = 0; pp < P; ++pp) {
-      const int v = vb + pp;
-      constexpr int dummy = 0; (void)dummy;
-      StreamRegs<K>& nxt = buf[(pp + 1) % P];
-      if (v < nsteps) {
-        consume(cur);
-        if (v + 1 < nsteps) decode_step<K>(nxt, hist, cur);
-      }
+      StreamRegs<K>& nxt = buf[(pp + 2) % P];
+      consume(cur, false);
+      decode_step<K>(nxt, hist, cur);
       prefetch(nxt);
     }
   }
+#pragma unroll
+  for (int pp = 0; pp < P; ++pp) {
+    if (v + pp < nsteps) {
+      consume(cur, true);
+      if (v + pp + 1 < nsteps) decode_step<K>(buf[(pp + 2) % P], hist, cur);
+    }
+  }
 
-  // ---- output side of the row blocks that end in this chunk (cur_seg of them)
-  __syncthreads();
-  const int nfin = cur_seg;
+  // ---- output side of the row blocks that end in this chunk (nfin of them): wave w takes (segment, activation row)
+  // pairs w, w + 8, ...
   const size_t slot_floats = (size_t)M * 128;
-  for (int idx = w; idx < nfin * M; idx += WG_WAVES) {
-    const int seg = idx / M, mrow = idx - seg * M, rb = rb_first + seg;
+  // row constants of the wave's first pair are fetched before the barrier: they do not depend on the partials
+  auto row_consts = [&](int rb, float& rs0, float& rs1, float& b0v, float& b1v) {
     const int r0 = rb * 128 + lane, r1 = r0 + 64;
-    const float rs0 = f16_bits_to_float(t.scales[r0]) * t.cbscale, rs1 = f16_bits_to_float(t.scales[r1]) * t.cbscale;
-    const float sg0 = sign_of(t.sv, r0), sg1 = sign_of(t.sv, r1);
-    float b0v = 0.f, b1v = 0.f;
+    rs0 = f16_bits_to_float(t.scales[r0]) * t.cbscale * INV_SQRT128;
+    rs1 = f16_bits_to_float(t.scales[r1]) * t.cbscale * INV_SQRT128;
+    b0v = 0.f; b1v = 0.f;
     if (t.bias != nullptr) { b0v = load_elem(t.bias, y_dtype, r0); b1v = load_elem(t.bias, y_dtype, r1); }
+    // output sign of rows lane and lane + 64 folded into the scale that is applied after the rotation
+    rs0 = sign_of(t.sv, r0) < 0.f ? -rs0 : rs0;
+    rs1 = sign_of(t.sv, r1) < 0.f ? -rs1 : rs1;
+  };
+  float f_rs0 = 0.f, f_rs1 = 0.f, f_b0 = 0.f, f_b1 = 0.f;
+  if (w < nfin * M) row_consts(rb_first + (M == 1 ? w : w / M), f_rs0, f_rs1, f_b0, f_b1);
+  __syncthreads();
+  for (int idx = w; idx < nfin * M; idx += WG_WAVES) {
+    const int seg = M == 1 ? idx : idx / M, mrow = idx - seg * M, rb = rb_first + seg;
+    const int r0 = rb * 128 + lane, r1 = r0 + 64;
+    float rs0 = f_rs0, rs1 = f_rs1, b0v = f_b0, b1v = f_b1;
+    if (idx != w) row_consts(rb, rs0, rs1, b0v, b1v);
     float v0s = 0.f, v1s = 0.f;
     bool failed = false;
     if (seg == 0 && c0 != 0) {
       // earlier chunks hold the beginning of this row block: chunks j0 .. blockIdx.x - 1, each in its own slot.  They
       // were dispatched before this workgroup, so waiting for them cannot deadlock; the wait is bounded all the same.
-      const int j0 = (rb * nblk) / chunk, j1 = (int)blockIdx.x;
+      // Eight contributors are read per round trip.
+      const int j0 = (int)(((unsigned long long)(unsigned)(rb * nblk) * t.chunk_magic) >> 40), j1 = (int)blockIdx.x;
       int tries = 0;
       for (;;) {
         bool missing = false;
         v0s = 0.f; v1s = 0.f;
-        for (int j = j0; j < j1; ++j) {
-          const uint32_t* pp = (const uint32_t*)(part + (size_t)j * slot_floats + (size_t)mrow * 128);
-          const uint32_t u0 = __hip_atomic_load(pp + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          const uint32_t u1 = __hip_atomic_load(pp + lane + 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          missing |= (u0 == 0u) | (u1 == 0u);
-          v0s += __uint_as_float(u0); v1s += __uint_as_float(u1);
+        for (int jb = j0; jb < j1; jb += 8) {
+          uint32_t u0[8], u1[8];
+#pragma unroll
+          for (int k = 0; k < 8; ++k) {
+            const int j = min(jb + k, j1 - 1);
+            const uint32_t* pp = (const uint32_t*)(part + (size_t)j * slot_floats + (size_t)mrow * 128);
+            u0[k] = __hip_atomic_load(pp + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            u1[k] = __hip_atomic_load(pp + lane + 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
+#pragma unroll
+          for (int k = 0; k < 8; ++k)
+            if (jb + k < j1) {
+              missing |= (u0[k] == 0u) | (u1[k] == 0u);
+              v0s += __uint_as_float(u0[k]); v1s += __uint_as_float(u1[k]);
+            }
         }
         if (!__any(missing)) break;
         if (++tries >= t.spin_limit) { failed = true; break; }
@@ -644,10 +707,11 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
     }
     const float* own = s_fin + ((size_t)seg * M + mrow) * 128;
     v0s += own[lane]; v1s += own[lane + 64];
-    v0s *= rs0; v1s *= rs1;
+    // the row scale applies before the output rotation; the sign and 1/sqrt(128) after it
+    v0s *= fabsf(rs0); v1s *= fabsf(rs1);
     fwht128_wave(v0s, v1s, lane);
-    v0s = v0s * INV_SQRT128 * sg0 + b0v;
-    v1s = v1s * INV_SQRT128 * sg1 + b1v;
+    v0s = __builtin_fmaf(v0s, rs0 < 0.f ? -1.f : 1.f, b0v);
+    v1s = __builtin_fmaf(v1s, rs1 < 0.f ? -1.f : 1.f, b1v);
     if (failed) { v0s = __builtin_nanf(""); v1s = v0s; }
     store_elem(t.y, y_dtype, (size_t)mrow * m + r0, v0s);
     store_elem(t.y, y_dtype, (size_t)mrow * m + r1, v1s);
@@ -792,6 +856,11 @@ inline size_t prerot_bytes(int n, int M) { return align256((size_t)M * n * 2) + 
 constexpr int NUM_CU = 256;
 constexpr int MAX_ROW_BLOCKS = 16384;
 constexpr int MAX_CHUNK = 4096;
+// the kernel divides step indices by n / 128 with a 40-bit reciprocal: exact while indices stay below 2^24
+inline bool shape_ok(int m, int n) {
+  return m > 0 && n > 0 && m % 128 == 0 && n % 128 == 0 && m / 128 <= MAX_ROW_BLOCKS && n / 128 < 65536 &&
+         (long)(m / 128) * (n / 128) < (1L << 24) - 2 * MAX_CHUNK;
+}
 
 inline bool plan_for_chunk(int m, int n, int M, int chunk, Plan& pl) {
   const int nblk = n / 128, rbs = m / 128;
@@ -857,6 +926,7 @@ inline size_t balanced_lds_request(size_t needed, int grid) {
 struct LinearLaunch {
   const uint32_t* qw; const void* x; const uint8_t* su; float* part;
   int m, n, M, chunk, flags;
+  unsigned long long nblk_magic;
   LinearTail tail;
 };
 
@@ -868,7 +938,7 @@ template <int K, int MB, bool PREROT> int launch_linear_v(const LinearLaunch& a,
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
   }
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(WG_THREADS), lds, st, a.qw, a.x, a.su, a.part, a.m, a.n, a.M, a.chunk, a.flags, a.tail);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(WG_THREADS), lds, st, a.qw, a.x, a.su, a.part, a.m, a.n, a.M, a.chunk, a.flags, a.nblk_magic, a.tail);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
   return HTR_OK;
@@ -925,7 +995,7 @@ int htr_abi_version(void) { return 1; }
 float htr_cbscale(void) { return (float)(1.0 / __builtin_sqrt(MEAN_SQ)); }
 
 size_t htr_workspace_bytes(int m, int n, int K, int M, int nsplit) {
-  if (K < 2 || K > 8 || m <= 0 || n <= 0 || m % 128 || n % 128 || m / 128 > MAX_ROW_BLOCKS || M < 1 || M > HTR_MAX_BATCH) return 0;
+  if (K < 2 || K > 8 || !shape_ok(m, n) || M < 1 || M > HTR_MAX_BATCH) return 0;
   Plan pl;
   if (!make_plan(m, n, M, nsplit, pl)) return 0;
   return WS_HEADER + PREROT_REGION + (size_t)pl.wgs * M * 128 * sizeof(float);
@@ -934,7 +1004,7 @@ size_t htr_workspace_bytes(int m, int n, int K, int M, int nsplit) {
 int htr_linear_plan(int m, int n, int K, int M, int nsplit, int* out6) {
   if (!out6) return HTR_ERR_NULL;
   if (K < 2 || K > 8) return HTR_ERR_K;
-  if (m <= 0 || n <= 0 || m % 128 || n % 128 || m / 128 > MAX_ROW_BLOCKS) return HTR_ERR_SHAPE;
+  if (!shape_ok(m, n)) return HTR_ERR_SHAPE;
   if (M < 1 || M > HTR_MAX_BATCH) return HTR_ERR_BATCH;
   Plan pl;
   if (!make_plan(m, n, M, nsplit, pl)) return HTR_ERR_SPLIT;
@@ -949,7 +1019,7 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
                size_t workspace_bytes, void* stream) {
   if (!qweight || !scales || !su || !sv || !x || !y) return HTR_ERR_NULL;
   if (K < 2 || K > 8) return HTR_ERR_K;
-  if (m <= 0 || n <= 0 || m % 128 || n % 128 || m / 128 > MAX_ROW_BLOCKS) return HTR_ERR_SHAPE;
+  if (!shape_ok(m, n)) return HTR_ERR_SHAPE;
   if (M < 1 || M > HTR_MAX_BATCH) return HTR_ERR_BATCH;
   if (!dtype_ok(x_dtype) || !dtype_ok(y_dtype)) return HTR_ERR_DTYPE;
   if (((uintptr_t)qweight & 15) || ((uintptr_t)scales & 1) || ((uintptr_t)x & (x_dtype == HTR_F32 ? 3 : 1)) ||
@@ -969,12 +1039,14 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
   a.qw = (const uint32_t*)qweight; a.x = x; a.su = (const uint8_t*)su;
   a.part = (float*)(wsp + PREROT_REGION);
   a.m = m; a.n = n; a.M = M; a.chunk = pl.chunk; a.flags = x_dtype | (y_dtype << 2);
+  a.nblk_magic = (((unsigned long long)1 << 40) + (unsigned)(n / 128) - 1) / (unsigned)(n / 128);
   LinearTail& t = a.tail;
   t.scales = (const uint16_t*)scales; t.sv = (const uint8_t*)sv; t.bias = bias; t.y = y;
   t.xt_g = nullptr; t.xs_g = nullptr; t.sc_g = nullptr;
   t.status = (uint32_t*)workspace;
   t.cbscale = htr_cbscale();
   t.spin_limit = g_spin_limit;
+  t.chunk_magic = (((unsigned long long)1 << 40) + (unsigned)pl.chunk - 1) / (unsigned)pl.chunk;
   hipStream_t st = (hipStream_t)stream;
   if (prerot) {
     t.xt_g = (const _Float16*)wsp;

@@ -292,12 +292,21 @@ __device__ __forceinline__ int scale_exponent(float amax) {
 __device__ __forceinline__ float pow2f(int e) { return __uint_as_float((uint32_t)(127 + e) << 23); }
 
 // Rotation of all activation rows ahead of the linear kernel (used where every workgroup rotating its own column
-// blocks would repeat too much work, and for float32 activations): one workgroup per row.
+// blocks would repeat too much work, and for float32 activations).  Workgroup (g, row) rotates column blocks
+// 8g .. 8g + 7 of one activation row, one block per wave; every workgroup scans the whole row for max|x| itself
+// (n / 512 loads per thread), which is cheaper than a second launch or an exchange between workgroups.
 __global__ __launch_bounds__(WG_THREADS) void k_rotate(const void* __restrict__ x, const uint8_t* __restrict__ su, int n, int x_dtype,
                                                        _Float16* __restrict__ xt_g, float* __restrict__ xs_g, float* __restrict__ sc_g) {
   __shared__ float s_max[WG_WAVES];
-  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, mrow = blockIdx.x, nblk = n >> 7;
+  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, mrow = blockIdx.y, nblk = n >> 7;
   const size_t row = (size_t)mrow * n;
+  const int blk = blockIdx.x * WG_WAVES + w;
+  const int col = blk * 128;
+  float va = 0.f, vb = 0.f;
+  if (blk < nblk) {                       // own block first: its loads overlap the scan
+    va = load_elem(x, x_dtype, row + col + lane) * sign_of(su, col + lane);
+    vb = load_elem(x, x_dtype, row + col + lane + 64) * sign_of(su, col + lane + 64);
+  }
   float mx = 0.f;
   for (int i = threadIdx.x; i < n; i += WG_THREADS) mx = fmaxf(mx, fabsf(load_elem(x, x_dtype, row + i)));
   mx = wave_max(mx);
@@ -308,11 +317,9 @@ __global__ __launch_bounds__(WG_THREADS) void k_rotate(const void* __restrict__ 
   for (int k = 0; k < WG_WAVES; ++k) amax = fmaxf(amax, s_max[k]);
   const int e = scale_exponent(amax);
   const float inv_sc = pow2f(-e);
-  if (threadIdx.x == 0) sc_g[mrow] = pow2f(e);
-  for (int blk = w; blk < nblk; blk += WG_WAVES) {
-    const int col = blk * 128;
-    float va = load_elem(x, x_dtype, row + col + lane) * sign_of(su, col + lane) * inv_sc;
-    float vb = load_elem(x, x_dtype, row + col + lane + 64) * sign_of(su, col + lane + 64) * inv_sc;
+  if (threadIdx.x == 0 && blockIdx.x == 0) sc_g[mrow] = pow2f(e);
+  if (blk < nblk) {
+    va *= inv_sc; vb *= inv_sc;
     fwht128_wave(va, vb, lane);
     const _Float16 ha = (_Float16)(va * INV_SQRT128), hb = (_Float16)(vb * INV_SQRT128);
     xt_g[row + col + lane] = ha;
@@ -345,7 +352,7 @@ template <int K> __device__ __forceinline__ void decode_step(const StreamRegs<K>
 // leaves the other P - 1 loads outstanding.
 #define HTR_PIN() __builtin_amdgcn_sched_barrier(0)
 
-template <int K, int MB, int P, bool PREROT>
+template <int K, int MB, int P, int D, bool PREROT>
 __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restrict__ qw, const void* __restrict__ x,
                                                        const uint8_t* __restrict__ su, float* __restrict__ part,
                                                        int m, int n, int M, int chunk, int flags,
@@ -462,12 +469,16 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
     }
   }
 
-  // ---- decode the first two steps into registers around the activation exchange: they need no x~, and they fill
-  // the time the other waves take to reach the barriers
+  // ---- decode the first D steps into registers around the activation exchange: they need no x~, and they fill the
+  // time the other waves take to reach the barriers (short chunks are decoded completely this way)
+  static_assert(D >= 2 && D <= P && D % 2 == 0, "pre-decoded steps come out of the first D stream buffers");
   const int hist = history_lane_byteaddr(lane);
-  DecodedStep<K> pre0, cur;
-  decode_step<K>(buf[0], hist, pre0);
-  prefetch(buf[0]);
+  DecodedStep<K> pre[D];
+#pragma unroll
+  for (int i = 0; i < D / 2; ++i) {
+    if (i == 0 || i < nsteps) decode_step<K>(buf[i], hist, pre[i]);
+    prefetch(buf[i]);
+  }
 
   if constexpr (!PREROT) {
     __syncthreads();
@@ -512,8 +523,11 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
       s_xs[i] = t.xs_g[((size_t)mrow * nblk + (pair_col(li) >> 7)) * 2 + (i & 1)];
     }
   }
-  if (nsteps > 1) decode_step<K>(buf[1 % P], hist, cur);
-  prefetch(buf[1 % P]);
+#pragma unroll
+  for (int i = D / 2; i < D; ++i) {
+    if (i < nsteps) decode_step<K>(buf[i], hist, pre[i]);
+    prefetch(buf[i]);
+  }
   __syncthreads();
 
   // ---- per-lane constants of the product and of the partial store
@@ -578,9 +592,10 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
     for (int mb = 0; mb < MB; ++mb) offs[mb] = __builtin_fmaf(k1534[mb], xsv[mb], offs[mb]);
     ++done; ++cur_blk; ++cur_li;
     const bool row_end = cur_blk == nblk;
-    const bool seg_end = row_end || (maybe_last && done == nsteps);
+    const bool last = maybe_last && done == nsteps;
+    const bool seg_end = row_end || last;
     if (row_end) { cur_blk = 0; if (all_blocks) cur_li = 0; }
-    if (!(maybe_last && done == nsteps)) load_b(cur_li);          // next step's operands (the slot exists: not the last step)
+    if (!last) load_b(cur_li);          // next step's operands (the slot exists: not the last step)
     if (seg_end) {
       // End of a segment: this wave's strip partial per activation row, the 1534 offset removed, the activation scale
       // undone, the two tile parities added (the parity-1 lane of a value is lane ^ 33).  A segment that ends its
@@ -623,12 +638,15 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
   // ---- main loop: one 128-column block (8 tiles of this wave's strip) per step.  Step v multiplies what the previous
   // step decoded, then decodes step v + 1 out of buffer (v + 1) % P while the matrix unit works, then refills it.
   // Groups of P steps that all have a successor run without bounds checks; the last steps are checked one by one.
-  consume(pre0, true);
-  int v = 1;
+#pragma unroll
+  for (int i = 0; i < D - 1; ++i)
+    if (i < nsteps) consume(pre[i], true);
+  DecodedStep<K> cur = pre[D - 1];
+  int v = D - 1;
   for (; v + P < nsteps; v += P) {
 #pragma unroll
     for (int pp = 0; pp < P; ++pp) {
-      StreamRegs<K>& nxt = buf[(pp + 2) % P];
+      StreamRegs<K>& nxt = buf[(pp + D) % P];
       consume(cur, false);
       decode_step<K>(nxt, hist, cur);
       prefetch(nxt);
@@ -638,7 +656,7 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
   for (int pp = 0; pp < P; ++pp) {
     if (v + pp < nsteps) {
       consume(cur, true);
-      if (v + pp + 1 < nsteps) decode_step<K>(buf[(pp + 2) % P], hist, cur);
+      if (v + pp + 1 < nsteps) decode_step<K>(buf[(pp + D) % P], hist, cur);
     }
   }
 
@@ -657,6 +675,7 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
     rs1 = sign_of(t.sv, r1) < 0.f ? -rs1 : rs1;
   };
   float f_rs0 = 0.f, f_rs1 = 0.f, f_b0 = 0.f, f_b1 = 0.f;
+  if (nfin == 0) return;        // a pure contributor: its partial is on its way, nothing else to do (uniform)
   if (w < nfin * M) row_consts(rb_first + (M == 1 ? w : w / M), f_rs0, f_rs1, f_b0, f_b1);
   __syncthreads();
   for (int idx = w; idx < nfin * M; idx += WG_WAVES) {
@@ -880,9 +899,11 @@ inline bool plan_for_chunk(int m, int n, int M, int chunk, Plan& pl) {
 }
 
 // Picks the chunk length (virtual steps per workgroup) with a cost model in microseconds fitted to chunk-length sweeps
-// on MI355X (K4): a fixed latency chain (launch, x fetch, rotation, partial exchange, output rotation), a per-step cost
-// that grows with the workgroups resident per CU, a penalty for chunks that do not tile the rows of column blocks,
-// the extra launch of a pre-rotation, and the slot reads of a finisher per contributor.
+// on MI355X (K4): a fixed latency chain (launch, x fetch, rotation, partial exchange, output rotation) that grows with
+// the contributors a finisher reads; a cost per step that depends on how many workgroups share a CU (one: latency
+// bound, cheaper on a part-filled chip, dearer for long chunks; several: throughput bound, proportional to the
+// load of the fullest CU); a penalty for chunks that do not tile the rows of column blocks; the extra launch of a
+// pre-rotation; and the growth of all per-step work with the number of activation rows.
 inline bool make_plan(int m, int n, int M, int nsplit, Plan& pl) {
   const int nblk = n / 128, rbs = m / 128;
   const long vtotal = (long)rbs * nblk;
@@ -894,6 +915,7 @@ inline bool make_plan(int m, int n, int M, int nsplit, Plan& pl) {
     return ok;
   }
   if (vtotal >= (long)64 * NUM_CU && nblk <= 64 && plan_for_chunk(m, n, M, nblk, pl)) return true;
+  const double rows = M <= 8 ? 1.0 + 0.065 * (M - 1) : (M <= 16 ? 2.2 : 6.5);
   double best = 1e30;
   bool found = false;
   const int max_chunk = (int)(vtotal < MAX_CHUNK ? vtotal : MAX_CHUNK);
@@ -901,12 +923,15 @@ inline bool make_plan(int m, int n, int M, int nsplit, Plan& pl) {
     Plan c;
     c.mb = pl.mb;
     if (!plan_for_chunk(m, n, M, chunk, c)) continue;
-    const double k = (double)c.wgs / NUM_CU;
-    const double waves = k <= 1.0 ? 1.0 : (double)((c.wgs + NUM_CU - 1) / NUM_CU);     // workgroups on the fullest CU
-    const double step = (waves <= 1.0 ? 0.55 : 0.42 * waves) * (1.0 + 0.25 * (pl.mb - 1));
+    const double fill = (double)c.wgs / NUM_CU;
     const bool aligned = (nblk % chunk == 0) || (chunk % nblk == 0);
     const int contributors = chunk >= nblk ? 1 : (nblk + chunk - 1) / chunk;
-    const double t = 4.5 + (c.prerot ? 2.5 : 0.0) + step * chunk * (aligned ? 1.0 : 1.15) + 0.05 * contributors;
+    const double steps = chunk * (aligned ? 1.0 : 1.08);
+    // one workgroup per CU or fewer: the chip works through `chunk` steps once; more: the fullest CU works through
+    // its workgroups one after the other, each with its own set-up and partial hand-over
+    const double body = fill <= 1.0 ? rows * (0.25 + 0.3 * fill + 0.008 * chunk) * steps
+                                    : fill * (rows * 0.6 * steps + 0.5 + 0.3 * M);
+    const double t = 4.5 + 0.06 * contributors + (c.prerot ? 3.0 : 0.0) + body;
     if (t < best) { best = t; pl = c; found = true; }
   }
   return found;
@@ -930,9 +955,10 @@ struct LinearLaunch {
   LinearTail tail;
 };
 
-template <int K, int MB, bool PREROT> int launch_linear_v(const LinearLaunch& a, int grid, size_t lds, hipStream_t st) {
+template <int K, int MB, bool DEEP, bool PREROT> int launch_linear_v(const LinearLaunch& a, int grid, size_t lds, hipStream_t st) {
   constexpr int P = K <= 4 ? 4 : (K <= 6 ? 3 : 2);          // wave-steps of weights in flight
-  auto kern = k_linear<K, MB, P, PREROT>;
+  constexpr int D = DEEP && P >= 4 ? 4 : 2;                 // steps decoded ahead of the activation exchange
+  auto kern = k_linear<K, MB, P, D, PREROT>;
   lds = balanced_lds_request(lds, grid);
   if (lds > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -943,11 +969,14 @@ template <int K, int MB, bool PREROT> int launch_linear_v(const LinearLaunch& a,
   if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
   return HTR_OK;
 }
+// Short chunks are decoded completely ahead of the activation exchange (more registers, so only for one activation
+// block and chunks whose prologue latency is a large part of the kernel); long chunks prefer occupancy.
 template <int K, bool PREROT> int launch_linear_kr(const LinearLaunch& a, int mb, int grid, size_t lds, hipStream_t st) {
+  const bool deep = a.chunk <= 8;
   switch (mb) {
-    case 1: return launch_linear_v<K, 1, PREROT>(a, grid, lds, st);
-    case 2: return launch_linear_v<K, 2, PREROT>(a, grid, lds, st);
-    default: return launch_linear_v<K, 4, PREROT>(a, grid, lds, st);
+    case 1: return deep ? launch_linear_v<K, 1, true, PREROT>(a, grid, lds, st) : launch_linear_v<K, 1, false, PREROT>(a, grid, lds, st);
+    case 2: return launch_linear_v<K, 2, false, PREROT>(a, grid, lds, st);
+    default: return launch_linear_v<K, 4, false, PREROT>(a, grid, lds, st);
   }
 }
 template <int K> int launch_linear_k(const LinearLaunch& a, bool prerot, int mb, int grid, size_t lds, hipStream_t st) {
@@ -1052,7 +1081,7 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
     t.xt_g = (const _Float16*)wsp;
     t.xs_g = (const float*)(wsp + align256((size_t)M * n * 2));
     t.sc_g = (const float*)(wsp + align256((size_t)M * n * 2) + align256((size_t)M * (n / 128) * 8));
-    hipLaunchKernelGGL(k_rotate, dim3(M), dim3(WG_THREADS), 0, st, x, (const uint8_t*)su, n, x_dtype, (_Float16*)t.xt_g,
+    hipLaunchKernelGGL(k_rotate, dim3((n / 128 + WG_WAVES - 1) / WG_WAVES, M), dim3(WG_THREADS), 0, st, x, (const uint8_t*)su, n, x_dtype, (_Float16*)t.xt_g,
                        (float*)t.xs_g, (float*)t.sc_g);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }

@@ -13,6 +13,7 @@ LIB_PATH = os.environ.get("HTR_GFX950_LIB") or os.path.join(_CSRC, "libhtr_gfx95
 
 BF16, F16, F32 = 0, 1, 2
 MAX_BATCH = 32
+MAX_GROUP = 4096
 
 _lib = None
 
@@ -26,6 +27,9 @@ SIGNATURES = {
     "htr_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "htr_linear_plan": (_i, [_i, _i, _i, _i, _i, ctypes.POINTER(ctypes.c_int)]),
     "htr_linear": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
+    "htr_grouped_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
+    "htr_linear_grouped": (_i, [_vp, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
+    "htr_set_spin_limit": (None, [_i]),
     "htr_decode_raw": (_i, [_vp, _vp, _i64, _i, _vp]),
     "htr_dequant_q": (_i, [_vp, _vp, _vp, _i, _i, _i, _vp]),
     "htr_dequant_w": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),

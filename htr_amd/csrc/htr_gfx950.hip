@@ -24,6 +24,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <string.h>
+#include <stdlib.h>
 
 #include "../../include/htr_gfx950.h"
 
@@ -263,6 +264,11 @@ struct LinearTail {
   unsigned long long chunk_magic;   // ceil(2^40 / chunk): step index -> chunk index
   float cbscale;
   int spin_limit;         // polls of the contributors' slots before a finisher gives up
+  // grouped launch (blockIdx.y = problem): per-problem pointers and row counts come from this device table, the
+  // pre-rotated activations and the partial slots of problem p start p strides into their regions
+  const htr_group_entry* group;
+  unsigned long long group_prerot_stride;   // bytes
+  unsigned long long group_part_stride;     // floats
 };
 
 constexpr int ROT_PAIRS = 16;  // (activation row, 128-column block) pairs a workgroup may rotate by itself
@@ -296,8 +302,18 @@ __device__ __forceinline__ float pow2f(int e) { return __uint_as_float((uint32_t
 // 8g .. 8g + 7 of one activation row, one block per wave; every workgroup scans the whole row for max|x| itself
 // (n / 512 loads per thread), which is cheaper than a second launch or an exchange between workgroups.
 __global__ __launch_bounds__(WG_THREADS) void k_rotate(const void* __restrict__ x, const uint8_t* __restrict__ su, int n, int x_dtype,
-                                                       _Float16* __restrict__ xt_g, float* __restrict__ xs_g, float* __restrict__ sc_g) {
+                                                       _Float16* __restrict__ xt_g, float* __restrict__ xs_g, float* __restrict__ sc_g,
+                                                       const htr_group_entry* __restrict__ group, unsigned long long group_stride) {
   __shared__ float s_max[WG_WAVES];
+  if (group != nullptr) {                  // grouped: blockIdx.z = problem, outputs shifted by the problem's stride
+    const htr_group_entry& ge = group[blockIdx.z];
+    if ((int)blockIdx.y >= ge.M) return;
+    x = ge.x; su = (const uint8_t*)ge.su;
+    const size_t shift = (size_t)blockIdx.z * group_stride;
+    xt_g = (_Float16*)((unsigned char*)xt_g + shift);
+    xs_g = (float*)((unsigned char*)xs_g + shift);
+    sc_g = (float*)((unsigned char*)sc_g + shift);
+  }
   const int lane = threadIdx.x & 63, w = threadIdx.x >> 6, mrow = blockIdx.y, nblk = n >> 7;
   const size_t row = (size_t)mrow * n;
   const int blk = blockIdx.x * WG_WAVES + w;
@@ -353,11 +369,29 @@ template <int K> __device__ __forceinline__ void decode_step(const StreamRegs<K>
 #define HTR_PIN() __builtin_amdgcn_sched_barrier(0)
 
 template <int K, int MB, int P, int D, bool PREROT>
-__global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restrict__ qw, const void* __restrict__ x,
-                                                       const uint8_t* __restrict__ su, float* __restrict__ part,
-                                                       int m, int n, int M, int chunk, int flags,
-                                                       unsigned long long nblk_magic, const LinearTail t) {
+__global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restrict__ qw_a, const void* __restrict__ x_a,
+                                                       const uint8_t* __restrict__ su_a, float* __restrict__ part_a,
+                                                       int m, int n, int M_a, int chunk, int flags,
+                                                       unsigned long long nblk_magic, const LinearTail t_a) {
   extern __shared__ __align__(16) unsigned char lds[];
+  const uint32_t* __restrict__ qw = qw_a;
+  const void* __restrict__ x = x_a;
+  const uint8_t* __restrict__ su = su_a;
+  float* __restrict__ part = part_a;
+  int M = M_a;
+  LinearTail t = t_a;
+  if (t_a.group != nullptr) {              // uniform: one entry of the problem table per blockIdx.y
+    const htr_group_entry& ge = t_a.group[blockIdx.y];
+    M = ge.M;
+    if (M <= 0) return;
+    qw = (const uint32_t*)ge.qweight; x = ge.x; su = (const uint8_t*)ge.su;
+    part = part_a + (size_t)blockIdx.y * t_a.group_part_stride;
+    t.scales = (const uint16_t*)ge.scales; t.sv = (const uint8_t*)ge.sv; t.bias = ge.bias; t.y = ge.y;
+    const size_t shift = (size_t)blockIdx.y * t_a.group_prerot_stride;
+    t.xt_g = (const _Float16*)((const unsigned char*)t_a.xt_g + shift);
+    t.xs_g = (const float*)((const unsigned char*)t_a.xs_g + shift);
+    t.sc_g = (const float*)((const unsigned char*)t_a.sc_g + shift);
+  }
   const int lane = threadIdx.x & 63;
   const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));   // wave index, provably uniform: keeps the
                                                                            // strip addressing on the scalar unit
@@ -950,7 +984,7 @@ inline size_t balanced_lds_request(size_t needed, int grid) {
 
 struct LinearLaunch {
   const uint32_t* qw; const void* x; const uint8_t* su; float* part;
-  int m, n, M, chunk, flags;
+  int m, n, M, chunk, flags, problems;
   unsigned long long nblk_magic;
   LinearTail tail;
 };
@@ -959,12 +993,12 @@ template <int K, int MB, bool DEEP, bool PREROT> int launch_linear_v(const Linea
   constexpr int P = K <= 4 ? 4 : (K <= 6 ? 3 : 2);          // wave-steps of weights in flight
   constexpr int D = DEEP && P >= 4 ? 4 : 2;                 // steps decoded ahead of the activation exchange
   auto kern = k_linear<K, MB, P, D, PREROT>;
-  lds = balanced_lds_request(lds, grid);
+  lds = balanced_lds_request(lds, grid * a.problems);
   if (lds > 48 * 1024) {
     hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
   }
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(WG_THREADS), lds, st, a.qw, a.x, a.su, a.part, a.m, a.n, a.M, a.chunk, a.flags, a.nblk_magic, a.tail);
+  hipLaunchKernelGGL(kern, dim3(grid, a.problems), dim3(WG_THREADS), lds, st, a.qw, a.x, a.su, a.part, a.m, a.n, a.M, a.chunk, a.flags, a.nblk_magic, a.tail);
   hipError_t e = hipGetLastError();
   if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
   return HTR_OK;
@@ -1067,7 +1101,7 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
   LinearLaunch a;
   a.qw = (const uint32_t*)qweight; a.x = x; a.su = (const uint8_t*)su;
   a.part = (float*)(wsp + PREROT_REGION);
-  a.m = m; a.n = n; a.M = M; a.chunk = pl.chunk; a.flags = x_dtype | (y_dtype << 2);
+  a.m = m; a.n = n; a.M = M; a.chunk = pl.chunk; a.flags = x_dtype | (y_dtype << 2); a.problems = 1;
   a.nblk_magic = (((unsigned long long)1 << 40) + (unsigned)(n / 128) - 1) / (unsigned)(n / 128);
   LinearTail& t = a.tail;
   t.scales = (const uint16_t*)scales; t.sv = (const uint8_t*)sv; t.bias = bias; t.y = y;
@@ -1075,6 +1109,7 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
   t.status = (uint32_t*)workspace;
   t.cbscale = htr_cbscale();
   t.spin_limit = g_spin_limit;
+  t.group = nullptr; t.group_prerot_stride = 0; t.group_part_stride = 0;
   t.chunk_magic = (((unsigned long long)1 << 40) + (unsigned)pl.chunk - 1) / (unsigned)pl.chunk;
   hipStream_t st = (hipStream_t)stream;
   if (prerot) {
@@ -1082,11 +1117,83 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
     t.xs_g = (const float*)(wsp + align256((size_t)M * n * 2));
     t.sc_g = (const float*)(wsp + align256((size_t)M * n * 2) + align256((size_t)M * (n / 128) * 8));
     hipLaunchKernelGGL(k_rotate, dim3((n / 128 + WG_WAVES - 1) / WG_WAVES, M), dim3(WG_THREADS), 0, st, x, (const uint8_t*)su, n, x_dtype, (_Float16*)t.xt_g,
-                       (float*)t.xs_g, (float*)t.sc_g);
+                       (float*)t.xs_g, (float*)t.sc_g, (const htr_group_entry*)nullptr, 0ull);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
   }
   HTR_FOR_K(K, return launch_linear_k<KK>(a, prerot, pl.mb, pl.wgs, pl.lds, st));
+  return HTR_OK;
+}
+
+// plan of a grouped launch: every problem has the same shape, so one plan serves all; the activations are always
+// rotated ahead (one launch for all problems) and the chunk is chosen for the whole grid
+static bool make_group_plan(int count, int m, int n, int max_M, Plan& pl) {
+  const int nblk = n / 128, rbs = m / 128;
+  const long vtotal = (long)rbs * nblk;
+  pl.mb = max_M <= 8 ? 1 : (max_M <= 16 ? 2 : 4);
+  // aim at a few workgroups per CU over all problems; chunks are whole rows of column blocks or divide one, so that
+  // no chunk straddles a row block; of those the one nearest the target (in ratio) that fits LDS
+  static const int per_cu = getenv("HTR_GROUP_WGS_PER_CU") ? atoi(getenv("HTR_GROUP_WGS_PER_CU")) : 4;
+  const double target = (double)vtotal * count / ((double)(per_cu > 0 ? per_cu : 4) * NUM_CU);
+  double best = 1e30;
+  bool found = false;
+  for (long chunk = 1; chunk <= vtotal && chunk <= MAX_CHUNK; ++chunk) {
+    if (chunk < nblk ? nblk % chunk != 0 : chunk % nblk != 0) continue;
+    Plan c;
+    c.mb = pl.mb;
+    if (!plan_for_chunk(m, n, max_M, (int)chunk, c)) continue;
+    const double ratio = chunk > target ? chunk / target : target / chunk;
+    if (ratio < best) { best = ratio; pl = c; found = true; }
+  }
+  pl.prerot = 1;
+  return found && prerot_bytes(n, max_M) <= PREROT_REGION;
+}
+
+size_t htr_grouped_workspace_bytes(int count, int m, int n, int K, int max_M) {
+  if (K < 2 || K > 8 || !shape_ok(m, n) || max_M < 1 || max_M > HTR_MAX_BATCH || count < 1 || count > HTR_MAX_GROUP) return 0;
+  Plan pl;
+  if (!make_group_plan(count, m, n, max_M, pl)) return 0;
+  return WS_HEADER + (size_t)count * prerot_bytes(n, max_M) + (size_t)count * pl.wgs * max_M * 128 * sizeof(float);
+}
+
+int htr_linear_grouped(const htr_group_entry* entries, int count, int m, int n, int K, int max_M, int x_dtype, int y_dtype,
+                       void* workspace, size_t workspace_bytes, void* stream) {
+  if (!entries) return HTR_ERR_NULL;
+  if (count < 1 || count > HTR_MAX_GROUP) return HTR_ERR_COUNT;
+  if (K < 2 || K > 8) return HTR_ERR_K;
+  if (!shape_ok(m, n)) return HTR_ERR_SHAPE;
+  if (max_M < 1 || max_M > HTR_MAX_BATCH) return HTR_ERR_BATCH;
+  if (!dtype_ok(x_dtype) || !dtype_ok(y_dtype)) return HTR_ERR_DTYPE;
+  if ((uintptr_t)entries & 7) return HTR_ERR_ALIGN;
+  Plan pl;
+  if (!make_group_plan(count, m, n, max_M, pl)) return HTR_ERR_SPLIT;
+  const size_t need = htr_grouped_workspace_bytes(count, m, n, K, max_M);
+  if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255)) return HTR_ERR_WORKSPACE;
+
+  unsigned char* wsp = (unsigned char*)workspace + WS_HEADER;
+  const size_t pre = prerot_bytes(n, max_M);
+  LinearLaunch a;
+  a.qw = nullptr; a.x = nullptr; a.su = nullptr;
+  a.part = (float*)(wsp + (size_t)count * pre);
+  a.m = m; a.n = n; a.M = max_M; a.chunk = pl.chunk; a.flags = x_dtype | (y_dtype << 2); a.problems = count;
+  a.nblk_magic = (((unsigned long long)1 << 40) + (unsigned)(n / 128) - 1) / (unsigned)(n / 128);
+  LinearTail& t = a.tail;
+  t.scales = nullptr; t.sv = nullptr; t.bias = nullptr; t.y = nullptr;
+  t.xt_g = (const _Float16*)wsp;
+  t.xs_g = (const float*)(wsp + align256((size_t)max_M * n * 2));
+  t.sc_g = (const float*)(wsp + align256((size_t)max_M * n * 2) + align256((size_t)max_M * (n / 128) * 8));
+  t.status = (uint32_t*)workspace;
+  t.cbscale = htr_cbscale();
+  t.spin_limit = g_spin_limit;
+  t.chunk_magic = (((unsigned long long)1 << 40) + (unsigned)pl.chunk - 1) / (unsigned)pl.chunk;
+  t.group = entries; t.group_prerot_stride = pre; t.group_part_stride = (unsigned long long)pl.wgs * max_M * 128;
+  hipStream_t st = (hipStream_t)stream;
+  hipLaunchKernelGGL(k_rotate, dim3((n / 128 + WG_WAVES - 1) / WG_WAVES, max_M, count), dim3(WG_THREADS), 0, st, (const void*)nullptr,
+                     (const uint8_t*)nullptr, n, x_dtype, (_Float16*)t.xt_g, (float*)t.xs_g, (float*)t.sc_g, entries,
+                     (unsigned long long)pre);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
+  HTR_FOR_K(K, return launch_linear_k<KK>(a, true, pl.mb, pl.wgs, pl.lds, st));
   return HTR_OK;
 }
 

@@ -88,6 +88,96 @@ def _linear_impl(x2, qweight, scales, su, sv, bias, out_dtype=None):
     return y
 
 
+def linear_grouped(xs, weights, biases=None, out_dtype=None):
+    """Many packed linears of one shape in one grouped launch: y_i = x_i @ W_i^T (+ bias_i).
+
+    xs: list of [M_i, n] tensors (M_i may be 0); weights: list of (qweight, scales, su, sv) of identical shapes and K;
+    returns the list of [M_i, m] results.  Routed experts are the use: the reference has no kernel for them and runs
+    one linear per expert (docs/ADAPTERS.md:19 of the reference), which on this GPU is dominated by launch latency.
+    Problems with more than LAUNCH_MAX_M rows are cut into several table entries.
+    """
+    if len(xs) != len(weights) or not xs:
+        raise RuntimeError("linear_grouped wants as many activation tensors as weight tuples, at least one")
+    m, n, K = wire.check_shapes(*weights[0])
+    dev = xs[0].device
+    if not xs[0].is_cuda:
+        raise RuntimeError("htr::linear runs on a ROCm device only; move the tensors to the GPU")
+    dt = xs[0].dtype
+    if dt not in _DTYPE_CODE:
+        raise KeyError(dt)
+    out_dtype = dt if out_dtype is None else out_dtype
+    rows = [int(x.shape[0]) for x in xs]
+    total = sum(rows)
+    y = torch.empty((total, m), dtype=out_dtype, device=dev)
+    outs, entries, keep = [], [], []
+    r = 0
+    for i, (x, w) in enumerate(zip(xs, weights)):
+        if wire.check_shapes(*w) != (m, n, K):
+            raise RuntimeError("linear_grouped: every problem must have the same m, n and K")
+        if x.dim() != 2 or x.shape[1] != n or x.dtype != dt or x.device != dev:
+            raise RuntimeError("linear_grouped: activations must be [M, n] tensors of one dtype on one device")
+        for t in w:
+            if t.device != dev or not t.is_contiguous():
+                raise RuntimeError("HTR-W1 tensors must be contiguous and on the device of x")
+        b = None if biases is None else biases[i]
+        if b is not None and (b.dtype != out_dtype or b.numel() != m or b.device != dev):
+            raise RuntimeError("bias must be [m] in the output dtype on the device of x")
+        xc = x.contiguous()
+        keep.append(xc)
+        outs.append(y[r:r + rows[i]])
+        for r0 in range(0, rows[i], LAUNCH_MAX_M):
+            mi = min(LAUNCH_MAX_M, rows[i] - r0)
+            entries.append([w[0].data_ptr(), w[1].data_ptr(), w[2].data_ptr(), w[3].data_ptr(),
+                            xc[r0:r0 + mi].data_ptr(), 0 if b is None else b.data_ptr(), y[r + r0:r + r0 + mi].data_ptr(), mi])
+        r += rows[i]
+    if not entries:
+        return outs
+    if len(entries) > _native.MAX_GROUP:
+        raise RuntimeError(f"linear_grouped: more than {_native.MAX_GROUP} table entries")
+    max_m = max(e[7] for e in entries)
+    L = _native.lib()
+    need = L.htr_grouped_workspace_bytes(len(entries), m, n, K, max_m)
+    if need == 0:
+        raise RuntimeError("libhtr_gfx950: no launch plan for this grouped shape")
+    with torch.cuda.device(dev):
+        stream = torch.cuda.current_stream(dev)
+        table = torch.tensor(entries, dtype=torch.int64).to(dev, non_blocking=False)       # 8 x int64 = one 64-byte entry
+        ws = workspace(dev, stream.cuda_stream, need)
+        _native.check(L.htr_linear_grouped(table.data_ptr(), len(entries), m, n, K, max_m, _DTYPE_CODE[dt],
+                                           _DTYPE_CODE[out_dtype], ws.data_ptr(), ws.numel(), stream.cuda_stream))
+    return outs
+
+
+def moe_experts(x, expert_ids, expert_weights, gate_up, down, activation=torch.nn.functional.silu):
+    """Routed-expert MLP on packed weights: y_t = sum_j w_tj * Down_e( act(Gate_e x_t) * Up_e x_t ), e = ids[t, j].
+
+    x [T, H]; expert_ids [T, top] integer; expert_weights [T, top]; gate_up[e] = HTR-W1 tuple of the fused [2F, H] matrix
+    (gate rows first), down[e] = HTR-W1 tuple of [H, F].  Two grouped launches cover all active experts; the result is
+    float32 [T, H].  The reference defines no such runtime (its experts are a composition of packed linears), so this
+    is that composition, batched.
+    """
+    T, H = x.shape
+    flat_e = expert_ids.reshape(-1)
+    order = torch.argsort(flat_e, stable=True)
+    tok = (order // expert_ids.shape[1])
+    counts = torch.bincount(flat_e, minlength=len(gate_up)).tolist()
+    xg = x[tok].contiguous()                                     # tokens grouped by expert
+    act = [e for e, c in enumerate(counts) if c]
+    offs, o = [], 0
+    for e in act:
+        offs.append(o)
+        o += counts[e]
+    h2 = linear_grouped([xg[o:o + counts[e]] for e, o in zip(act, offs)], [gate_up[e] for e in act], out_dtype=torch.float32)
+    F = h2[0].shape[1] // 2
+    hid = torch.cat(h2, 0)
+    hid = (activation(hid[:, :F]) * hid[:, F:]).to(x.dtype).contiguous()
+    out = linear_grouped([hid[o:o + counts[e]] for e, o in zip(act, offs)], [down[e] for e in act], out_dtype=torch.float32)
+    wflat = expert_weights.reshape(-1)[order].to(torch.float32)
+    y = torch.zeros((T, H), dtype=torch.float32, device=x.device)
+    y.index_add_(0, tok, torch.cat(out, 0) * wflat[:, None])
+    return y
+
+
 @torch.library.custom_op("htr::linear", mutates_args=())
 def htr_linear_op(x2: torch.Tensor, qweight: torch.Tensor, scales: torch.Tensor, su: torch.Tensor, sv: torch.Tensor,
                   bias: torch.Tensor | None) -> torch.Tensor:

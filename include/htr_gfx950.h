@@ -56,10 +56,12 @@ int htr_abi_version(void);
 float htr_cbscale(void);
 
 /*
- * Bytes of zero-initialised device workspace htr_linear needs for this problem (counters +
- * split partials).  The caller allocates it once, zeroes it once, and may reuse it for any
- * later call whose requirement is not larger, as long as calls that share a workspace are
- * ordered on one stream: kernels leave the counter words zero on exit.
+ * Bytes of zero-initialised device workspace htr_linear needs for this problem (a status
+ * word, room for pre-rotated activations, one partial slot per workgroup).  The caller
+ * allocates it once, zeroes it once, and may reuse it for any later call whose requirement
+ * is not larger, as long as calls that share a workspace are ordered on one stream: kernels
+ * leave the partial slots zero on exit.  The first 32-bit word stays zero unless a kernel
+ * gave up waiting for a partial (see htr_set_spin_limit).
  * Reference: the per-device int32[65536] counter tensor (htr/ops.py:24-28) plus the
  * `part` tensors the extension allocates per call (htr/csrc/htr_kernels.cu:1145).
  * nsplit: as in htr_linear.
@@ -67,10 +69,11 @@ float htr_cbscale(void);
 size_t htr_workspace_bytes(int m, int n, int K, int M, int nsplit);
 
 /*
- * The launch plan htr_linear would use: out6 = {column splits, 128-column blocks per split, row blocks per
- * workgroup, workgroups, 1 if finishers are elected by counter, dynamic LDS bytes}.  No reference counterpart as a
- * function; it exposes what nsplit_for / fused_nsplit decide there (htr/ops.py:31-45).
- * nsplit: 0 = library policy; otherwise (row blocks per workgroup << 16) | column splits, either part 0 = search.
+ * The launch plan htr_linear would use: out6 = {steps (128x128 weight blocks of one row block, walked row-major)
+ * per workgroup, workgroups, row blocks that can end inside one workgroup's chunk, distinct column blocks per
+ * workgroup, 1 if the activations are rotated by a launch of their own, dynamic LDS bytes}.  No reference counterpart
+ * as a function; it exposes what nsplit_for / fused_nsplit decide there (htr/ops.py:31-45).
+ * nsplit: 0 = library policy; otherwise the steps per workgroup (bit 30 set: force the separate rotation launch).
  */
 int htr_linear_plan(int m, int n, int K, int M, int nsplit, int* out6);
 
@@ -83,11 +86,47 @@ int htr_linear_plan(int m, int n, int K, int M, int nsplit, int* out6);
  *   bias   [m] in y_dtype, or NULL
  *   y      [M, m] row-major, y_dtype
  *   nsplit 0 = library policy; otherwise an explicit plan as in htr_linear_plan (tuning)
+ *   x must be 4-byte aligned for the in-kernel rotation; other 2-byte aligned bf16/f16 rows take the rotation launch
  */
 int htr_linear(const void* qweight, const void* scales, const void* su, const void* sv,
                const void* x, const void* bias, void* y,
                int m, int n, int K, int M, int x_dtype, int y_dtype, int nsplit,
                void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * One entry of a grouped launch: the HTR-W1 tensors, activations and output of one problem.  The table lives in
+ * DEVICE memory (so that a routing kernel can fill it), is 8-byte aligned and is read by the kernels only.
+ */
+typedef struct {
+  const void* qweight;
+  const void* scales;
+  const void* su;
+  const void* sv;
+  const void* x;      /* [M, n] row-major, 4-byte aligned */
+  const void* bias;   /* [m] in the output type, or NULL */
+  void* y;            /* [M, m] row-major */
+  int32_t M;          /* activation rows of this problem, 0 .. max_M (0 = skip) */
+  int32_t reserved;
+} htr_group_entry;
+
+/*
+ * `count` packed linears of ONE shape (m, n, K) in two launches (activation rotation for all problems, then the fused
+ * decode-product-epilogue for all problems): routed experts, whose per-expert launches would each pay the full launch
+ * latency for a few microseconds of work.  No counterpart in the reference, which has no runtime kernel for routed
+ * experts and composes them from per-expert linears (docs/ADAPTERS.md:19); the per-problem result is that of
+ * htr_linear on the same tensors.  max_M bounds the rows of any problem (1 .. HTR_MAX_BATCH).
+ * Workspace: htr_grouped_workspace_bytes() bytes, zeroed once, same rules as for htr_linear.
+ */
+size_t htr_grouped_workspace_bytes(int count, int m, int n, int K, int max_M);
+int htr_linear_grouped(const htr_group_entry* entries_device, int count, int m, int n, int K, int max_M,
+                       int x_dtype, int y_dtype, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Polls (about a microsecond each) a finishing workgroup waits for the partials of earlier workgroups before it gives
+ * up, stores NaN for its rows and sets bit 0 of the first workspace word.  Default 2^20.  No counterpart in the
+ * reference; exists so that the bounded wait can be exercised.
+ */
+void htr_set_spin_limit(int polls);
 
 /*
  * Integer decode, tile order: out[tile, t] = v(s_t) as int16, tile = ti*(n/16)+tj, t = 16r+c.

@@ -278,6 +278,57 @@ def test_moe_expert_stack_top6_of_64(dev, oracle):
     assert _rel(got, y_ref) <= 4e-3, _rel(got, y_ref)
 
 
+def test_grouped_launch_matches_single_launches(dev, oracle):
+    """Grouped launch against per-problem launches (bit-identical partial order is not promised: compare to the oracle
+    and to the single launches within tolerance), ragged row counts including 0 and more than one launch's worth."""
+    from htr_amd import ops, wire
+    print("grouped launch", flush=True)
+    m, n, K = 384, 512, 4
+    rows = [3, 0, 1, 16, 40, 7]
+    ws = [wire.synth_linear(m, n, K, 900 + i) for i in range(len(rows))]
+    xs = [wire.synth_activation(max(r, 1), n, 950 + i)[:r] for i, r in enumerate(rows)]
+    bias = [torch.randn(m, generator=torch.Generator().manual_seed(i)).float() if i % 2 else None for i in range(len(rows))]
+    got = ops.linear_grouped([x.to(dev) for x in xs], [tuple(t.to(dev) for t in w) for w in ws],
+                             [None if b is None else b.to(dev) for b in bias], out_dtype=torch.float32)
+    for i, r in enumerate(rows):
+        assert tuple(got[i].shape) == (r, m)
+        if r == 0:
+            continue
+        ref = _ref(oracle, *ws[i], xs[i], bias[i])
+        assert _rel(got[i].cpu().numpy(), ref) <= REL_TOL, (i, _rel(got[i].cpu().numpy(), ref))
+        one = ops.linear_f32out(xs[i].to(dev), *[t.to(dev) for t in ws[i]], None if bias[i] is None else bias[i].to(dev))
+        assert float((one - got[i]).abs().max()) <= 2e-4 * float(one.abs().max())
+
+
+def test_moe_64_experts_grouped(dev, oracle):
+    """BASELINE configuration 5, all 64 experts materialised: gate/up 1408x2048 (fused to 2816x2048) and down 2048x1408
+    at K4, top-6 routing of 16 tokens with seeded softmax-routed ids; two grouped launches against the per-expert
+    composition on the CPU oracle."""
+    from htr_amd import ops, wire
+    print("moe 64 experts grouped", flush=True)
+    E, T, TOP, H, F = 64, 16, 6, 2048, 1408
+    g = torch.Generator().manual_seed(20261125 + 5000)
+    probs = torch.softmax(torch.randn(T, E, generator=g), dim=-1)
+    w, ids = torch.topk(probs, TOP, dim=-1)
+    x = torch.randn(T, H, generator=g).bfloat16()
+    gate_up = [wire.synth_linear(2 * F, H, 4, 7000 + e) for e in range(E)]
+    down = [wire.synth_linear(H, F, 4, 7100 + e) for e in range(E)]
+    y = ops.moe_experts(x.to(dev), ids.to(dev), w.to(dev), [tuple(t.to(dev) for t in p) for p in gate_up],
+                        [tuple(t.to(dev) for t in p) for p in down]).cpu().numpy()
+    y_ref = np.zeros((T, H))
+    for e in range(E):
+        tok, slot = torch.nonzero(ids == e, as_tuple=True)
+        if tok.numel() == 0:
+            continue
+        r2 = oracle.c_linear(x[tok].float().numpy(), *[t.numpy() for t in gate_up[e]])
+        rh = torch.from_numpy(r2).float()
+        rh = (torch.nn.functional.silu(rh[:, :F]) * rh[:, F:]).bfloat16().float().numpy()
+        ro = oracle.c_linear(rh, *[t.numpy() for t in down[e]])
+        np.add.at(y_ref, tok.numpy(), ro * w[tok, slot].numpy().astype(np.float64)[:, None])
+    # two chained linears with a bf16 rounding between them (see test_moe_expert_stack_top6_of_64)
+    assert _rel(y, y_ref) <= 4e-3, _rel(y, y_ref)
+
+
 def test_lm_head_shape(dev, oracle):
     from htr_amd import ops
     print("lm_head 152064x4096", flush=True)

@@ -897,12 +897,18 @@ int g_spin_limit = 1 << 20;     // polls (about a microsecond each) before a fin
 
 struct Plan { int chunk, wgs, segfin, nbl, mb, prerot; size_t lds; };
 
-// Workspace: [256-byte header: status word][pre-rotated activations, fixed region][one partial slot per workgroup].
-// Partial slots must be all-zero between calls, and no call may leave other data where a later call of another shape
-// expects such slots: hence the fixed region in front of them.
+// Workspace: two halves, split at workspace_bytes / 2 (rounded down to 256).  First half: [256-byte header: status
+// word][one partial slot per workgroup]; it must be all-zero between calls.  Second half: scratch for the pre-rotated
+// activations, left as it is.  The split depends only on the size the caller passes, not on the problem, so no call can
+// leave scratch data where a later call of another shape expects zeroed slots (as long as the caller passes the same
+// size with the same buffer).
 constexpr size_t WS_HEADER = 256;
-constexpr size_t PREROT_REGION = (size_t)4 << 20;
 inline size_t align256(size_t v) { return (v + 255) / 256 * 256; }
+inline size_t ws_need(size_t slot_bytes, size_t scratch_bytes) {
+  const size_t a = align256(WS_HEADER + slot_bytes), b = align256(scratch_bytes);
+  return 2 * (a > b ? a : b);
+}
+inline size_t ws_half(size_t workspace_bytes) { return workspace_bytes / 2 / 256 * 256; }
 // bytes of the pre-rotated activations, their block sums and the row scales
 inline size_t prerot_bytes(int n, int M) { return align256((size_t)M * n * 2) + align256((size_t)M * (n / 128) * 8) + align256((size_t)M * 4); }
 
@@ -928,7 +934,6 @@ inline bool plan_for_chunk(int m, int n, int M, int chunk, Plan& pl) {
   // a workgroup rotates its own column blocks while that is at most ROT_PAIRS (row, block) pairs; beyond that the
   // activations are rotated once, ahead of the launch
   pl.prerot = M * pl.nbl > ROT_PAIRS ? 1 : 0;
-  if (pl.prerot && prerot_bytes(n, M) > PREROT_REGION) return false;
   return true;
 }
 
@@ -945,7 +950,7 @@ inline bool make_plan(int m, int n, int M, int nsplit, Plan& pl) {
   if (nsplit > 0) {                                                 // explicit plan (tuning): chunk length in the low
     const int chunk = nsplit & 0xFFFFF;                             // 20 bits, bit 30 = force pre-rotation
     bool ok = chunk > 0 ? plan_for_chunk(m, n, M, chunk, pl) : false;
-    if (ok && (nsplit & (1 << 30))) { if (prerot_bytes(n, M) <= PREROT_REGION) pl.prerot = 1; else ok = false; }
+    if (ok && (nsplit & (1 << 30))) pl.prerot = 1;
     return ok;
   }
   if (vtotal >= (long)64 * NUM_CU && nblk <= 64 && plan_for_chunk(m, n, M, nblk, pl)) return true;
@@ -1061,7 +1066,7 @@ size_t htr_workspace_bytes(int m, int n, int K, int M, int nsplit) {
   if (K < 2 || K > 8 || !shape_ok(m, n) || M < 1 || M > HTR_MAX_BATCH) return 0;
   Plan pl;
   if (!make_plan(m, n, M, nsplit, pl)) return 0;
-  return WS_HEADER + PREROT_REGION + (size_t)pl.wgs * M * 128 * sizeof(float);
+  return ws_need((size_t)pl.wgs * M * 128 * sizeof(float), prerot_bytes(n, M));
 }
 
 int htr_linear_plan(int m, int n, int K, int M, int nsplit, int* out6) {
@@ -1093,14 +1098,13 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
   // the in-kernel rotation reads 16-bit elements in pairs: float32 activations, and rows that do not start on a
   // 4-byte boundary, take the pre-rotation
   const bool prerot = pl.prerot || x_dtype == HTR_F32 || ((uintptr_t)x & 3);
-  if (prerot && prerot_bytes(n, M) > PREROT_REGION) return HTR_ERR_SPLIT;
   const size_t need = htr_workspace_bytes(m, n, K, M, nsplit);
   if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255)) return HTR_ERR_WORKSPACE;
 
-  unsigned char* wsp = (unsigned char*)workspace + WS_HEADER;
+  unsigned char* wsp = (unsigned char*)workspace + ws_half(workspace_bytes);      // scratch half
   LinearLaunch a;
   a.qw = (const uint32_t*)qweight; a.x = x; a.su = (const uint8_t*)su;
-  a.part = (float*)(wsp + PREROT_REGION);
+  a.part = (float*)((unsigned char*)workspace + WS_HEADER);
   a.m = m; a.n = n; a.M = M; a.chunk = pl.chunk; a.flags = x_dtype | (y_dtype << 2); a.problems = 1;
   a.nblk_magic = (((unsigned long long)1 << 40) + (unsigned)(n / 128) - 1) / (unsigned)(n / 128);
   LinearTail& t = a.tail;
@@ -1146,14 +1150,14 @@ static bool make_group_plan(int count, int m, int n, int max_M, Plan& pl) {
     if (ratio < best) { best = ratio; pl = c; found = true; }
   }
   pl.prerot = 1;
-  return found && prerot_bytes(n, max_M) <= PREROT_REGION;
+  return found;
 }
 
 size_t htr_grouped_workspace_bytes(int count, int m, int n, int K, int max_M) {
   if (K < 2 || K > 8 || !shape_ok(m, n) || max_M < 1 || max_M > HTR_MAX_BATCH || count < 1 || count > HTR_MAX_GROUP) return 0;
   Plan pl;
   if (!make_group_plan(count, m, n, max_M, pl)) return 0;
-  return WS_HEADER + (size_t)count * prerot_bytes(n, max_M) + (size_t)count * pl.wgs * max_M * 128 * sizeof(float);
+  return ws_need((size_t)count * pl.wgs * max_M * 128 * sizeof(float), (size_t)count * prerot_bytes(n, max_M));
 }
 
 int htr_linear_grouped(const htr_group_entry* entries, int count, int m, int n, int K, int max_M, int x_dtype, int y_dtype,
@@ -1170,11 +1174,11 @@ int htr_linear_grouped(const htr_group_entry* entries, int count, int m, int n, 
   const size_t need = htr_grouped_workspace_bytes(count, m, n, K, max_M);
   if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255)) return HTR_ERR_WORKSPACE;
 
-  unsigned char* wsp = (unsigned char*)workspace + WS_HEADER;
+  unsigned char* wsp = (unsigned char*)workspace + ws_half(workspace_bytes);      // scratch half
   const size_t pre = prerot_bytes(n, max_M);
   LinearLaunch a;
   a.qw = nullptr; a.x = nullptr; a.su = nullptr;
-  a.part = (float*)(wsp + (size_t)count * pre);
+  a.part = (float*)((unsigned char*)workspace + WS_HEADER);
   a.m = m; a.n = n; a.M = max_M; a.chunk = pl.chunk; a.flags = x_dtype | (y_dtype << 2); a.problems = count;
   a.nblk_magic = (((unsigned long long)1 << 40) + (unsigned)(n / 128) - 1) / (unsigned)(n / 128);
   LinearTail& t = a.tail;

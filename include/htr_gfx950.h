@@ -62,6 +62,10 @@ float htr_cbscale(void);
  * is not larger, as long as calls that share a workspace are ordered on one stream: kernels
  * leave the partial slots zero on exit.  The first 32-bit word stays zero unless a kernel
  * gave up waiting for a partial (see htr_set_spin_limit).
+ * The library splits the buffer at workspace_bytes / 2: the first half holds the status word and the
+ * partial slots (the part that must be zero), the second half is scratch.  Pass the same
+ * workspace_bytes whenever you pass the same buffer, so that the split stays where it was;
+ * htr_linear and htr_linear_grouped may then share one buffer.
  * Reference: the per-device int32[65536] counter tensor (htr/ops.py:24-28) plus the
  * `part` tensors the extension allocates per call (htr/csrc/htr_kernels.cu:1145).
  * nsplit: as in htr_linear.

@@ -288,6 +288,10 @@ def test_grouped_launch_matches_single_launches(dev, oracle):
     ws = [wire.synth_linear(m, n, K, 900 + i) for i in range(len(rows))]
     xs = [wire.synth_activation(max(r, 1), n, 950 + i)[:r] for i, r in enumerate(rows)]
     bias = [torch.randn(m, generator=torch.Generator().manual_seed(i)).float() if i % 2 else None for i in range(len(rows))]
+    # a launch with pre-rotated activations of another shape first: the scratch it leaves in the shared workspace must
+    # not be mistaken for partials by the grouped launch (or by the single launches after it)
+    big = _case(256, 4096, 4, 24, 123)
+    ops.linear_f32out(big[4].to(dev), *[t.to(dev) for t in big[:4]])
     got = ops.linear_grouped([x.to(dev) for x in xs], [tuple(t.to(dev) for t in w) for w in ws],
                              [None if b is None else b.to(dev) for b in bias], out_dtype=torch.float32)
     for i, r in enumerate(rows):

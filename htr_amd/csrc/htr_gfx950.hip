@@ -4,9 +4,12 @@
 //   v(s) = bytesum((s * 0xDF6ADF + 0x34983) mod 2^32) - 510              (docs/FORMAT.md:7-13 of the reference)
 //
 // Work decomposition of the fused linear kernel
-//   workgroup = 8 waves = one 128-row output block (one H128 output block) x one split of the input columns
+//   step      = one 128-row x 128-column block of the weight; the steps of a linear, row-major, are cut into equal
+//               contiguous chunks, one workgroup each, so the workgroup count does not depend on the shape
+//   workgroup = 8 waves = the 8 strips of a 128-row block (one H128 output block)
 //   wave      = one 16-row strip of tiles; per step it streams the 8 consecutive tiles that cover one 128-column
-//               input block (8 * 32K contiguous bytes: each lane loads its 4K contiguous bytes)
+//               input block (8 * 32K contiguous bytes: each lane loads its 4K contiguous bytes) through a buffer
+//               descriptor that covers exactly its bytes of the chunk, so loads beyond the end cost nothing
 //   lane      = (tile-in-step = lane / 8, row pair q = lane % 8): the K dwords a lane loads are exactly the stream
 //               bits of tile rows 2q and 2q+1 (32 steps); the 16-K history bits come from the previous lane's last
 //               dword through the LDS crossbar (ds_bpermute), the tail-biting wrap is lane 7 -> lane 0 of the tile
@@ -19,8 +22,9 @@
 //               the even tiles in MFMA column 2r and the odd tiles in column 2r + 1, and only D[i][2r + h(i)] is
 //               kept.  Eight activation rows share one MFMA; more rows reuse the decoded A registers.
 //   offset    = the constant 1534 is removed afterwards with 1534 * sum(x~) per activation row.
-//   epilogue  = split partials meet in a workspace; the last workgroup of a row block (arrival counter) sums them in
-//               a fixed order, applies scale * CBSCALE, the output H128, sv, bias and the cast.
+//   epilogue  = the workgroup whose chunk holds the last step of a row block finishes it: it adds the partials the
+//               earlier chunks of that row block left in their workspace slots (fixed order) to its own, applies
+//               scale * CBSCALE, the output H128, sv, bias and the cast.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <string.h>
@@ -965,11 +969,13 @@ inline bool make_plan(int m, int n, int M, int nsplit, Plan& pl) {
     const double fill = (double)c.wgs / NUM_CU;
     const bool aligned = (nblk % chunk == 0) || (chunk % nblk == 0);
     const int contributors = chunk >= nblk ? 1 : (nblk + chunk - 1) / chunk;
-    const double steps = chunk * (aligned ? 1.0 : 1.08);
+    const double steps = chunk * (aligned ? 1.0 : 1.03);
     // one workgroup per CU or fewer: the chip works through `chunk` steps once; more: the fullest CU works through
     // its workgroups one after the other, each with its own set-up and partial hand-over
+    // (a grid slightly above one workgroup per CU leaves a few CUs with two: it costs nearly as much as two everywhere)
+    const double fill2 = fill < 1.5 ? 1.5 : fill;
     const double body = fill <= 1.0 ? rows * (0.25 + 0.3 * fill + 0.008 * chunk) * steps
-                                    : fill * (rows * 0.6 * steps + 0.5 + 0.3 * M);
+                                    : fill2 * (rows * 0.6 * steps + 0.5 + 0.3 * M);
     const double t = 4.5 + 0.06 * contributors + (c.prerot ? 3.0 : 0.0) + body;
     if (t < best) { best = t; pl = c; found = true; }
   }

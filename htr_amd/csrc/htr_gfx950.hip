@@ -367,6 +367,22 @@ template <int K> __device__ __forceinline__ void decode_step(const StreamRegs<K>
   d.a[0] = win.template group8<0>();
 }
 
+// The same with something to do at the fence between the two parts (a barrier and LDS reads, in the batched kernel)
+template <int K, typename F> __device__ __forceinline__ void decode_step_mid(const StreamRegs<K>& r, int hist, DecodedStep<K>& d, F&& mid) {
+  const uint32_t prev = (uint32_t)__builtin_amdgcn_ds_bpermute(hist, (int)r.d[K - 1]);
+  __builtin_amdgcn_sched_barrier(0);
+  Window<K> win;
+  win.build_tail(r);
+  d.a[1] = win.template group8<8>();
+  d.a[2] = win.template group8<16>();
+  __builtin_amdgcn_sched_barrier(0);
+  mid();
+  __builtin_amdgcn_sched_barrier(0);
+  d.a[3] = win.template group8<24>();
+  win.build_head(prev);
+  d.a[0] = win.template group8<0>();
+}
+
 // Nothing may move across a weight-stream load: the loads of a wave must issue in program order, one per step, so
 // that the number of loads in flight behind any buffer is the same on every path and the wait in front of a decode
 // leaves the other P - 1 loads outstanding.
@@ -775,6 +791,244 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
   }
 }
 
+// ------------------------------------------------------------------------------------------------ batched linear
+// Variant for 8 .. 32 activation rows.  With that many rows the rotated activations of a whole chunk no longer fit in
+// LDS next to useful chunk lengths, and short chunks mean that every workgroup copies a large activation slice and
+// hands over a large partial for little weight traffic.  Here a workgroup owns one 128-row block and 1/S of its
+// column blocks (grid = S x row blocks), and the activations (rotated ahead by k_rotate) are staged through LDS one
+// 128-column block at a time, double-buffered, one barrier per step; the decoded weights of a step feed MB * 4 matrix
+// instructions.  The split S along the columns is only as large as filling the chip needs; S = 1 needs no exchange.
+template <int K, int MB, int P>
+__global__ __launch_bounds__(WG_THREADS) void k_linear_batch(const uint32_t* __restrict__ qw, float* __restrict__ part,
+                                                             int m, int n, int M, int S, int flags, const LinearTail t) {
+  extern __shared__ __align__(16) unsigned char lds[];
+  const int lane = threadIdx.x & 63;
+  const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int nblk = n >> 7;
+  const int s_idx = blockIdx.x, rb = blockIdx.y;
+  const int cb = (nblk + S - 1) / S;                               // column blocks per split
+  const int c_begin = s_idx * cb, c_end = min(nblk, c_begin + cb);
+  const int nsteps = c_end - c_begin;                              // >= 1: the host picks S so that no split is empty
+  const int y_dtype = (flags >> 2) & 3;
+
+  // LDS: [2 buffers][(M + 1) rows][144 halves] x~ blocks, [2][2 M] sums, [M][128] partials of the finishing workgroup
+  constexpr int ROWH = 128 + 16;
+  const int bufh = (M + 1) * ROWH;
+  _Float16* xt = (_Float16*)lds;
+  float* s_xs = (float*)(lds + (size_t)2 * bufh * 2);
+  float* s_fin = s_xs + 4 * M;
+
+  // ---- activation staging: thread = one 16-byte piece (8 halves) of the block: row tid / 16, piece tid % 16
+  const int tid = threadIdx.x;
+  const bool has_piece = tid < M * 16, has_sum = tid < 2 * M;
+  const int p_row = tid >> 4, p_idx = tid & 15;
+  const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)t.xt_g, 0, M * n * 2, 0x00020000);
+  const __amdgpu_buffer_rsrc_t srsrc = __builtin_amdgcn_make_buffer_rsrc((void*)t.xs_g, 0, M * nblk * 8, 0x00020000);
+  constexpr int OUT_OF_RANGE = 0x7FFFFF00;
+  const int piece_lds = p_row * ROWH + (p_idx & 1) * 64 + (p_idx >> 1) * 8;        // halves, inside a buffer
+  // Blocks travel two steps ahead of their use in two register sets (q = block parity): loads return in order, so
+  // waiting for a block also waits for every weight load issued before it, and one step of distance would cut the
+  // weight stream's run-ahead to a single step.
+  u4 xg[2];
+  float xsg[2];
+  auto stage_load = [&](int blk, int q) {    // block index in the row; beyond the split: zeros, no traffic
+    HTR_PIN();
+    const bool live = blk < c_end;
+    xg[q] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, live && has_piece ? (p_row * n + blk * 128 + p_idx * 8) * 2 : OUT_OF_RANGE, 0, 0);
+    xsg[q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(srsrc, live && has_sum ? (((tid >> 1) * nblk + blk) * 2 + (tid & 1)) * 4 : OUT_OF_RANGE, 0, 0));
+    HTR_PIN();
+  };
+  auto stage_store = [&](int q) {            // block of parity q goes to buffer q
+    if (has_piece) *(u4*)(xt + q * bufh + piece_lds) = xg[q];
+    if (has_sum) s_xs[q * 2 * M + tid] = xsg[q];
+  };
+  for (int i = tid; i < ROWH / 2; i += WG_THREADS) {               // zero rows of both buffers
+    ((uint32_t*)(xt + (size_t)M * ROWH))[i] = 0u;
+    ((uint32_t*)(xt + bufh + (size_t)M * ROWH))[i] = 0u;
+  }
+  stage_load(c_begin, 0);
+  stage_load(c_begin + 1, 1);
+
+  // ---- the weight stream of this wave: one contiguous piece of its strip
+  constexpr int STEP_BYTES = 256 * K;
+  const uint32_t* wave_base = qw + ((size_t)(rb * 8 + w) * nblk + (size_t)c_begin) * (STEP_BYTES / 4);
+  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)wave_base, 0, nsteps * STEP_BYTES, 0x00020000);
+  int pf_off = lane * 4 * K;
+  StreamRegs<K> buf[P];
+  auto prefetch = [&](StreamRegs<K>& dst) {
+    HTR_PIN();
+    load_stream_buffer<K>(rsrc, pf_off, dst);
+    pf_off += STEP_BYTES;
+    HTR_PIN();
+  };
+#pragma unroll
+  for (int p = 0; p < P; ++p) prefetch(buf[p]);
+
+  // ---- per-lane constants of the product (as in k_linear)
+  const int g = lane >> 4, n16 = lane & 15;
+  const int par = g >> 1;
+  const bool mine = (n16 & 1) == par;
+  int boff[MB], xsoff[MB];
+  float sc[MB], offs[MB], k1534[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    const int mrow = mb * 8 + (n16 >> 1);
+    const bool live = mine && mrow < M;
+    boff[mb] = (mrow < M ? mrow : M) * ROWH + 8 * (2 * g + (n16 & 1));
+    xsoff[mb] = live ? 2 * mrow + par : -1;
+    offs[mb] = 0.f;
+    sc[mb] = live ? t.sc_g[mrow] : 0.f;
+    k1534[mb] = live ? 1534.f : 0.f;
+  }
+  f4 acc[MB][2];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) { acc[mb][0] = f4{0.f, 0.f, 0.f, 0.f}; acc[mb][1] = f4{0.f, 0.f, 0.f, 0.f}; }
+
+  h8 B0[MB], B1[MB];
+  float xsv[MB];
+  auto load_b = [&](int bsel) {
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      const _Float16* bp = xt + bsel * bufh + boff[mb];
+      B0[mb] = *(const h8*)bp;
+      B1[mb] = *(const h8*)(bp + 64);
+      xsv[mb] = s_xs[bsel * 2 * M + max(xsoff[mb], 0)];
+    }
+  };
+
+  // step 0: its block goes to buffer 0, the block of step 2 is requested, the first weights are decoded meanwhile
+  static_assert(P % 2 == 0, "the block parity of a step must be static in the unrolled loop");
+  const int hist = history_lane_byteaddr(lane);
+  stage_store(0);
+  stage_load(c_begin + 2, 0);
+  DecodedStep<K> cur;
+  decode_step<K>(buf[0], hist, cur);
+  prefetch(buf[0]);
+  __syncthreads();
+  load_b(0);
+
+  auto multiply = [&](const DecodedStep<K>& d) {
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) acc[mb][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[0], B0[mb], acc[mb][0], 0, 0, 0);
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) acc[mb][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[2], B0[mb], acc[mb][1], 0, 0, 0);
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) acc[mb][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[1], B1[mb], acc[mb][0], 0, 0, 0);
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) acc[mb][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[3], B1[mb], acc[mb][1], 0, 0, 0);
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) offs[mb] = __builtin_fmaf(k1534[mb], xsv[mb], offs[mb]);
+  };
+  // One step with a successor: multiply step v, put the block of step v + 1 (in registers since the previous step)
+  // into the other buffer, request the block of step v + 2, decode step v + 1; between the two halves of the decode
+  // the workgroup meets, after which the B operands of step v + 1 are read (their latency hides behind the rest).
+  auto step_with_next = [&](int v, int q, StreamRegs<K>& nxt) {      // q = (v + 1) & 1, static
+    multiply(cur);
+    stage_store(q);
+    stage_load(c_begin + v + 3, q);
+    decode_step_mid<K>(nxt, hist, cur, [&]() { __syncthreads(); load_b(q); });
+    prefetch(nxt);
+  };
+  int v = 0;
+  for (; v + P < nsteps; v += P) {
+#pragma unroll
+    for (int pp = 0; pp < P; ++pp) step_with_next(v + pp, (pp + 1) & 1, buf[(pp + 1) % P]);
+  }
+#pragma unroll
+  for (int pp = 0; pp < P; ++pp) {
+    if (v + pp + 1 < nsteps) step_with_next(v + pp, (pp + 1) & 1, buf[(pp + 1) % P]);
+    else if (v + pp < nsteps) multiply(cur);
+  }
+
+  // ---- this wave's strip partial per activation row: offset removed, activation scale undone, tile parities added
+  const bool finisher = s_idx == S - 1;
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    const int mrow = mb * 8 + (n16 >> 1);
+    float tot[8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int rr = 0; rr < 2; ++rr) {
+        const float val = xsoff[mb] >= 0 ? (acc[mb][rr][j] - offs[mb]) * sc[mb] : 0.f;
+        float lo_half, hi_half;
+        halves32(lane_xor_dpp<1>(val), lo_half, hi_half);
+        tot[2 * j + rr] = val + hi_half;
+      }
+    if (lane < 32 && (n16 & 1) == 0 && mrow < M) {
+      const int rowi = 16 * w + 8 * (g & 1);
+      if (finisher) {
+        float* dst = s_fin + (size_t)mrow * 128 + rowi;
+        *(f4*)dst = f4{tot[0], tot[1], tot[2], tot[3]};
+        *(f4*)(dst + 4) = f4{tot[4], tot[5], tot[6], tot[7]};
+      } else {
+        uint32_t* dst = (uint32_t*)(part + (((size_t)rb * S + s_idx) * M + mrow) * 128 + rowi);
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          __hip_atomic_store(dst + i, __float_as_uint(tot[i]) | 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+  }
+  if (!finisher) return;
+
+  // ---- output side: the last split of the row block adds the other splits' partials (fixed order) and finishes
+  const int r0 = rb * 128 + lane, r1 = r0 + 64;
+  float rs0 = f16_bits_to_float(t.scales[r0]) * t.cbscale * INV_SQRT128;
+  float rs1 = f16_bits_to_float(t.scales[r1]) * t.cbscale * INV_SQRT128;
+  const float sg0 = sign_of(t.sv, r0), sg1 = sign_of(t.sv, r1);
+  float b0v = 0.f, b1v = 0.f;
+  if (t.bias != nullptr) { b0v = load_elem(t.bias, y_dtype, r0); b1v = load_elem(t.bias, y_dtype, r1); }
+  __syncthreads();
+  for (int mrow = w; mrow < M; mrow += WG_WAVES) {
+    float v0s = 0.f, v1s = 0.f;
+    bool failed = false;
+    if (S > 1) {
+      int tries = 0;
+      for (;;) {
+        bool missing = false;
+        v0s = 0.f; v1s = 0.f;
+        for (int jb = 0; jb < S - 1; jb += 8) {
+          uint32_t u0[8], u1[8];
+#pragma unroll
+          for (int k = 0; k < 8; ++k) {
+            const int j = min(jb + k, S - 2);
+            const uint32_t* pp = (const uint32_t*)(part + (((size_t)rb * S + j) * M + mrow) * 128);
+            u0[k] = __hip_atomic_load(pp + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            u1[k] = __hip_atomic_load(pp + lane + 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
+#pragma unroll
+          for (int k = 0; k < 8; ++k)
+            if (jb + k < S - 1) {
+              missing |= (u0[k] == 0u) | (u1[k] == 0u);
+              v0s += __uint_as_float(u0[k]); v1s += __uint_as_float(u1[k]);
+            }
+        }
+        if (!__any(missing)) break;
+        if (++tries >= t.spin_limit) { failed = true; break; }
+        __builtin_amdgcn_s_sleep(2);
+      }
+      if (!failed) {
+        for (int j = 0; j < S - 1; ++j) {
+          uint32_t* pp = (uint32_t*)(part + (((size_t)rb * S + j) * M + mrow) * 128);
+          __hip_atomic_store(pp + lane, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_store(pp + lane + 64, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      } else if (lane == 0) {
+        __hip_atomic_fetch_or(t.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    const float* own = s_fin + (size_t)mrow * 128;
+    v0s += own[lane]; v1s += own[lane + 64];
+    v0s *= rs0; v1s *= rs1;
+    fwht128_wave(v0s, v1s, lane);
+    v0s = __builtin_fmaf(v0s, sg0, b0v);
+    v1s = __builtin_fmaf(v1s, sg1, b1v);
+    if (failed) { v0s = __builtin_nanf(""); v1s = v0s; }
+    store_elem(t.y, y_dtype, (size_t)mrow * m + r0, v0s);
+    store_elem(t.y, y_dtype, (size_t)mrow * m + r1, v1s);
+  }
+}
+
 // ------------------------------------------------------------------------------------------------ debug decodes
 template <int K, int U> struct ForEach32 {
   template <typename F> __device__ __forceinline__ static void run(const Window<K>& w, F&& f) {
@@ -1028,6 +1282,52 @@ template <int K> int launch_linear_k(const LinearLaunch& a, bool prerot, int mb,
   return prerot ? launch_linear_kr<K, true>(a, mb, grid, lds, st) : launch_linear_kr<K, false>(a, mb, grid, lds, st);
 }
 
+// ---- batched kernel: split S of the column blocks per row block
+struct BatchPlan { int S, cb, wgs, mb; size_t lds; };
+constexpr int BATCH_MIN_M = 8;      // rows from which the library policy takes the batched kernel
+inline size_t batch_lds_bytes(int M) { return (size_t)2 * (M + 1) * (128 + 16) * 2 + (size_t)4 * M * 4 + (size_t)M * 128 * 4; }
+inline bool make_batch_plan(int m, int n, int M, int want_S, BatchPlan& bp) {
+  const int nblk = n / 128, rbs = m / 128;
+  bp.mb = M <= 8 ? 1 : (M <= 16 ? 2 : 4);
+  bp.lds = batch_lds_bytes(M);
+  // Measured on MI355X (K4, 8..32 rows, 4096..28672 output rows): one workgroup per CU is the best fill; every further
+  // split adds partial traffic that grows with the rows.  So: the largest split that keeps the grid within the CU
+  // count, among the splits that leave no column range empty.
+  const int limit = want_S > 0 ? want_S : (NUM_CU / rbs > 1 ? NUM_CU / rbs : 1);
+  bool found = false;
+  for (int S = 1; S <= nblk && S <= limit; ++S) {
+    const int cb = (nblk + S - 1) / S;
+    if ((nblk + cb - 1) / cb != S) continue;                       // some split would be empty
+    if (want_S > 0 && S != want_S) continue;
+    bp.S = S; bp.cb = cb; bp.wgs = rbs * S; found = true;
+  }
+  return found;
+}
+
+template <int K, int MB> int launch_batch_v(const uint32_t* qw, float* part, int m, int n, int M, int flags, const LinearTail& t,
+                                            const BatchPlan& bp, hipStream_t st) {
+  auto kern = k_linear_batch<K, MB, 4>;
+  size_t lds = balanced_lds_request(bp.lds, bp.wgs);
+  if (lds > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
+  }
+  hipLaunchKernelGGL(kern, dim3(bp.S, m / 128), dim3(WG_THREADS), lds, st, qw, part, m, n, M, bp.S, flags, t);
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
+  return HTR_OK;
+}
+template <int K> int launch_batch_k(const uint32_t* qw, float* part, int m, int n, int M, int flags, const LinearTail& t,
+                                    const BatchPlan& bp, hipStream_t st) {
+  switch (bp.mb) {
+    case 1: return launch_batch_v<K, 1>(qw, part, m, n, M, flags, t, bp, st);
+    case 2: return launch_batch_v<K, 2>(qw, part, m, n, M, flags, t, bp, st);
+    default: return launch_batch_v<K, 4>(qw, part, m, n, M, flags, t, bp, st);
+  }
+}
+// nsplit bit 29: batched kernel with the split in the low bits (0 = policy); otherwise the policy decides by M
+inline bool wants_batch(int M, int nsplit) { return nsplit > 0 ? (nsplit & (1 << 29)) != 0 : M >= BATCH_MIN_M; }
+
 #define HTR_FOR_K(K, EXPR)                 \
   switch (K) {                             \
     case 2: { constexpr int KK = 2; EXPR; } break; \
@@ -1070,6 +1370,11 @@ float htr_cbscale(void) { return (float)(1.0 / __builtin_sqrt(MEAN_SQ)); }
 
 size_t htr_workspace_bytes(int m, int n, int K, int M, int nsplit) {
   if (K < 2 || K > 8 || !shape_ok(m, n) || M < 1 || M > HTR_MAX_BATCH) return 0;
+  if (wants_batch(M, nsplit)) {
+    BatchPlan bp;
+    if (!make_batch_plan(m, n, M, nsplit > 0 ? nsplit & 0xFFFFF : 0, bp)) return 0;
+    return ws_need((size_t)bp.wgs * M * 128 * sizeof(float), prerot_bytes(n, M));
+  }
   Plan pl;
   if (!make_plan(m, n, M, nsplit, pl)) return 0;
   return ws_need((size_t)pl.wgs * M * 128 * sizeof(float), prerot_bytes(n, M));
@@ -1080,6 +1385,12 @@ int htr_linear_plan(int m, int n, int K, int M, int nsplit, int* out6) {
   if (K < 2 || K > 8) return HTR_ERR_K;
   if (!shape_ok(m, n)) return HTR_ERR_SHAPE;
   if (M < 1 || M > HTR_MAX_BATCH) return HTR_ERR_BATCH;
+  if (wants_batch(M, nsplit)) {
+    BatchPlan bp;
+    if (!make_batch_plan(m, n, M, nsplit > 0 ? nsplit & 0xFFFFF : 0, bp)) return HTR_ERR_SPLIT;
+    out6[0] = bp.cb; out6[1] = bp.wgs; out6[2] = 1; out6[3] = 1; out6[4] = 1; out6[5] = (int)bp.lds;
+    return HTR_OK;
+  }
   Plan pl;
   if (!make_plan(m, n, M, nsplit, pl)) return HTR_ERR_SPLIT;
   out6[0] = pl.chunk; out6[1] = pl.wgs; out6[2] = pl.segfin; out6[3] = pl.nbl; out6[4] = pl.prerot; out6[5] = (int)pl.lds;
@@ -1099,6 +1410,32 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
   if (((uintptr_t)qweight & 15) || ((uintptr_t)scales & 1) || ((uintptr_t)x & (x_dtype == HTR_F32 ? 3 : 1)) ||
       ((uintptr_t)y & (y_dtype == HTR_F32 ? 3 : 1)) || (bias && ((uintptr_t)bias & (y_dtype == HTR_F32 ? 3 : 1))))
     return HTR_ERR_ALIGN;
+  if (wants_batch(M, nsplit)) {
+    BatchPlan bp;
+    if (!make_batch_plan(m, n, M, nsplit > 0 ? nsplit & 0xFFFFF : 0, bp)) return HTR_ERR_SPLIT;
+    const size_t need = htr_workspace_bytes(m, n, K, M, nsplit);
+    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255)) return HTR_ERR_WORKSPACE;
+    unsigned char* wsp = (unsigned char*)workspace + ws_half(workspace_bytes);
+    LinearTail t;
+    t.scales = (const uint16_t*)scales; t.sv = (const uint8_t*)sv; t.bias = bias; t.y = y;
+    t.xt_g = (const _Float16*)wsp;
+    t.xs_g = (const float*)(wsp + align256((size_t)M * n * 2));
+    t.sc_g = (const float*)(wsp + align256((size_t)M * n * 2) + align256((size_t)M * (n / 128) * 8));
+    t.status = (uint32_t*)workspace;
+    t.cbscale = htr_cbscale();
+    t.spin_limit = g_spin_limit;
+    t.chunk_magic = 0;
+    t.group = nullptr; t.group_prerot_stride = 0; t.group_part_stride = 0;
+    hipStream_t st = (hipStream_t)stream;
+    hipLaunchKernelGGL(k_rotate, dim3((n / 128 + WG_WAVES - 1) / WG_WAVES, M), dim3(WG_THREADS), 0, st, x, (const uint8_t*)su, n, x_dtype,
+                       (_Float16*)t.xt_g, (float*)t.xs_g, (float*)t.sc_g, (const htr_group_entry*)nullptr, 0ull);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
+    float* part = (float*)((unsigned char*)workspace + WS_HEADER);
+    const int flags = x_dtype | (y_dtype << 2);
+    HTR_FOR_K(K, return launch_batch_k<KK>((const uint32_t*)qweight, part, m, n, M, flags, t, bp, st));
+    return HTR_OK;
+  }
   Plan pl;
   if (!make_plan(m, n, M, nsplit, pl)) return HTR_ERR_SPLIT;
   // the in-kernel rotation reads 16-bit elements in pairs: float32 activations, and rows that do not start on a

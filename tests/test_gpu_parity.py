@@ -93,12 +93,12 @@ def test_dequant_w_original_basis(dev, oracle, K):
 
 def test_prefill_path_dequant_then_gemm(dev, oracle):
     from htr_amd import ops
-    print("prefill M=96", flush=True)
-    qw, sc, su, sv, x = _case(512, 384, 4, 96, 808)
+    print("prefill M=160", flush=True)
+    qw, sc, su, sv, x = _case(512, 384, 4, 160, 808)
     bias = torch.randn(512, generator=torch.Generator().manual_seed(2)).bfloat16()
-    assert 96 > ops.GEMV_LOOP_MAX
+    assert 160 > ops.GEMV_LOOP_MAX
     y = ops.linear(x.to(dev), *[t.to(dev) for t in (qw, sc, su, sv)], bias.to(dev))
-    assert y.dtype == torch.bfloat16 and tuple(y.shape) == (96, 512)
+    assert y.dtype == torch.bfloat16 and tuple(y.shape) == (160, 512)
     ref = _ref(oracle, qw, sc, su, sv, x, bias)
     # bf16 weights and bf16 output: compare at bf16 resolution of the largest magnitudes
     assert _rel(y.float().cpu().numpy(), ref) <= 2.0 ** -6
@@ -118,7 +118,7 @@ def test_linear_f32_out_within_tolerance(dev, oracle, K, M, shape):
     assert _rel(y, ref) <= REL_TOL, _rel(y, ref)
 
 
-@pytest.mark.parametrize("K,M", [(3, 16), (4, 9), (4, 16), (4, 32), (3, 32), (5, 17), (4, 45)])
+@pytest.mark.parametrize("K,M", [(3, 16), (4, 9), (4, 16), (4, 32), (3, 32), (5, 17), (4, 45), (4, 100), (2, 8), (8, 24)])
 def test_linear_small_batch_blocks(dev, oracle, K, M):
     from htr_amd import ops
     print(f"linear batch K={K} M={M}", flush=True)

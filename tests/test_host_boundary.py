@@ -70,14 +70,22 @@ def test_launch_plan_is_consistent(L, m, n, M):
     assert L.htr_linear_plan(m, n, 4, M, 0, out) == 0
     chunk, wgs, segfin, nbl, prerot, lds = list(out)
     nblk, rbs = n // 128, m // 128
+    need = L.htr_workspace_bytes(m, n, 4, M, 0)
+    assert need >= 256 + wgs * M * 128 * 4                                       # header + one partial slot per workgroup
+    if M >= 8:
+        # batched kernel: `chunk` column blocks per split, S = ceil(nblk / chunk) splits per row block, no empty split,
+        # activations always rotated ahead
+        S = -(-nblk // chunk)
+        assert wgs == rbs * S and (S - 1) * chunk < nblk and prerot == 1 and lds <= 64 * 1024
+        # an explicit split is honoured (bit 29 selects the batched kernel)
+        assert L.htr_linear_plan(m, n, 4, M, (1 << 29) | 1, out) == 0 and out[0] == nblk and out[1] == rbs
+        return
     assert chunk >= 1 and (wgs - 1) * chunk < rbs * nblk <= wgs * chunk          # chunks tile the step space exactly
     assert nbl == min(chunk, nblk) and lds <= 64 * 1024
     assert segfin == (chunk + nblk - 1) // nblk                                  # row blocks that can end inside one chunk
     assert prerot == (1 if M * nbl > 16 else 0)                                  # a workgroup rotates at most 16 pairs itself
-    need = L.htr_workspace_bytes(m, n, 4, M, 0)
-    assert need >= 256 + wgs * M * 128 * 4                                       # header + one partial slot per workgroup
     # an explicit chunk length is honoured
-    assert L.htr_linear_plan(m, n, 4, M, 1, out) == 0 or M * 128 * 2 > 60000
+    assert L.htr_linear_plan(m, n, 4, M, 1, out) == 0
     if out[0] == 1:
         assert out[1] == rbs * nblk
 

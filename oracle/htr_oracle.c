@@ -373,3 +373,77 @@ void htr_o_set_num_threads(int t) {
   (void)t;
 #endif
 }
+
+/* ------------------------------------------------------------------------------------------------ encoder search
+ * Batched bitshift-trellis Viterbi, restated from htr/reference.py:6-50 of the reference: minimises
+ * sum_t w[t] * (x[t] - cb[s_t])^2 over state sequences with s_t = ((s_{t-1} << K) & mask) | bits, L-bit states
+ * (L = 16 in the codec; smaller L exists so that tests can compare with an exhaustive search).  Two passes when
+ * tailbite: the first fixes j0 = argmin(final cost) & (Sj - 1); the second admits at t = 0 only the states whose
+ * upper part is j0 and at the end only the states whose lower part is j0, which makes the stream circular.
+ * Arithmetic is float32 in the reference's order: d = (x - cb)^2, cost = m + w * d; every min / argmin takes the
+ * FIRST index among equal values (htr/reference.py:29, 37, 41).  states: [B, T] uint32.  Returns 0, or -1 on
+ * allocation failure. */
+static int viterbi_pass(const float* x, const float* w, const float* cb, int L, int K, int T, int use_j0, uint32_t j0,
+                        float* cost, float* m, uint8_t* bps) {
+  const uint32_t S = 1u << L, nb = 1u << K, Sj = S >> K;
+  for (uint32_t s = 0; s < S; ++s) {                                   /* htr/reference.py:22-27 */
+    const float diff = x[0] - cb[s];
+    const float d0 = w[0] * (diff * diff);
+    cost[s] = (use_j0 && (s >> K) != j0) ? INFINITY : d0;
+  }
+  for (int t = 1; t < T; ++t) {                                        /* htr/reference.py:29-33 */
+    for (uint32_t low = 0; low < Sj; ++low) {
+      float best = cost[low];
+      uint32_t bi = 0;
+      for (uint32_t j = 1; j < nb; ++j) {
+        const float c = cost[j * Sj + low];
+        if (c < best) { best = c; bi = j; }
+      }
+      m[low] = best;
+      bps[(size_t)(t - 1) * Sj + low] = (uint8_t)bi;
+    }
+    for (uint32_t low = 0; low < Sj; ++low)
+      for (uint32_t b = 0; b < nb; ++b) {
+        const uint32_t s = low * nb + b;
+        const float diff = x[t] - cb[s];
+        const float d = diff * diff;
+        cost[s] = m[low] + w[t] * d;
+      }
+  }
+  return 0;
+}
+
+int htr_o_viterbi(const float* x, const float* w, const float* cb, int L, int K, int T, int64_t B, int tailbite,
+                  uint32_t* states) {
+  const uint32_t S = 1u << L, Sj = S >> K;
+  int fail = 0;
+#pragma omp parallel for schedule(dynamic)
+  for (int64_t b = 0; b < B; ++b) {
+    float* cost = (float*)malloc(sizeof(float) * S);
+    float* m = (float*)malloc(sizeof(float) * Sj);
+    uint8_t* bps = (uint8_t*)malloc((size_t)(T > 1 ? T - 1 : 1) * Sj);
+    if (!cost || !m || !bps) { fail = 1; free(cost); free(m); free(bps); continue; }
+    const float* xb = x + b * T;
+    const float* wb = w + b * T;
+    viterbi_pass(xb, wb, cb, L, K, T, 0, 0, cost, m, bps);
+    if (tailbite) {                                                    /* htr/reference.py:35-40 */
+      uint32_t a = 0;
+      for (uint32_t s = 1; s < S; ++s) if (cost[s] < cost[a]) a = s;
+      const uint32_t j0 = a & (Sj - 1);
+      viterbi_pass(xb, wb, cb, L, K, T, 1, j0, cost, m, bps);
+      for (uint32_t s = 0; s < S; ++s) if ((s & (Sj - 1)) != j0) cost[s] = INFINITY;
+    }
+    uint32_t s = 0;                                                    /* htr/reference.py:41-49 */
+    for (uint32_t q = 1; q < S; ++q) if (cost[q] < cost[s]) s = q;
+    uint32_t* st = states + b * T;
+    st[T - 1] = s;
+    for (int t = T - 1; t > 0; --t) {
+      const uint32_t low = s >> K;
+      const uint32_t top = bps[(size_t)(t - 1) * Sj + low];
+      s = top * Sj + low;
+      st[t - 1] = s;
+    }
+    free(cost); free(m); free(bps);
+  }
+  return fail ? -1 : 0;
+}

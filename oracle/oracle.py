@@ -14,8 +14,10 @@ __graft_entry__.py and the cpu_baseline leg of bench.py do, and only as the chec
 All functions are pinned by known-answer tests in tests/test_oracle_kat.py that were not
 produced by this code: generator/codebook constants from the closed form, the reference
 test-suite's string bit-oracle construction (tests/test_release.py:28-38 of the reference),
-sign byte 170 (:40-43), Hadamard orthogonality (:45-47), hand-made streams.  No function
-here is "parity unpinned".
+sign byte 170 (:40-43), Hadamard orthogonality (:45-47), hand-made streams.  The encoder search
+(c_viterbi) is pinned by exhaustive search on small trellises, by the stream invariants of the reference's own
+test (tests/test_release.py:12-19) and by vectors the reference's function produced (tests/golden/viterbi.npz).
+No function here is "parity unpinned".
 """
 import ctypes
 import math
@@ -304,6 +306,26 @@ def c_decode_then_matmul_f32(x, qweight, scales, su8, sv8):
     lib().htr_o_matmul_xwT_f32(_p(xf), _p(W), ctypes.c_int(xf.shape[0]), ctypes.c_int64(W.shape[0]),
                                ctypes.c_int64(W.shape[1]), _p(y))
     return y
+
+
+def c_viterbi(x, w, K, cb=None, L=16, tailbite=True):
+    """Tail-biting bitshift-trellis Viterbi (htr/reference.py:6-50): x, w float32 [B, T] -> states uint32 [B, T].
+    cb: [2^L] float32 state values (default: the RDNA24 codebook, L = 16)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    if cb is None:
+        cb = c_codebook_f32()
+    cb = np.ascontiguousarray(cb, dtype=np.float32)
+    assert cb.size == 1 << L and x.shape == w.shape and x.ndim == 2
+    B, T = x.shape
+    out = np.empty((B, T), dtype=np.uint32)
+    f = lib().htr_o_viterbi
+    f.restype = ctypes.c_int
+    f.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                  ctypes.c_int64, ctypes.c_int, ctypes.c_void_p]
+    rc = f(_p(x), _p(w), _p(cb), L, K, T, B, 1 if tailbite else 0, _p(out))
+    assert rc == 0
+    return out
 
 
 def c_num_threads():

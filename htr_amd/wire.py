@@ -30,6 +30,69 @@ def gen_values(states):
     return ((x & 0xFF) + ((x >> 8) & 0xFF) + ((x >> 16) & 0xFF) + ((x >> 24) & 0xFF)) - 510
 
 
+_CACHE = {}
+
+
+def codebook_f32(device="cpu"):
+    """cb[s] = float32(v(s) / rms), rms = sqrt(mean v^2) in float64 (htr/wire.py:19-25 of the reference)."""
+    key = ("cb", str(device))
+    if key not in _CACHE:
+        v = gen_values(torch.arange(S, dtype=torch.int64)).double()
+        _CACHE[key] = (v / math.sqrt(SUM_V_SQ / S)).float().to(device)
+    return _CACHE[key]
+
+
+def hadamard(n, device="cpu"):
+    """Sylvester Hadamard matrix / sqrt(n), built in float64 and rounded once to float32 (htr/wire.py:80-87)."""
+    key = ("had", n, str(device))
+    if key not in _CACHE:
+        h = torch.ones(1, 1, dtype=torch.float64)
+        while h.shape[0] < n:
+            h = torch.cat([torch.cat([h, h], 1), torch.cat([h, -h], 1)], 0)
+        _CACHE[key] = (h / math.sqrt(n)).float().to(device)
+    return _CACHE[key]
+
+
+def blk_had_cols_T(W, bs=RHT_BLOCK):
+    """Every block of bs consecutive columns of W times H (htr/wire.py:90-92)."""
+    m, n = W.shape
+    return (W.reshape(m, n // bs, bs) @ hadamard(bs, W.device)).reshape(m, n)
+
+
+def unpack_states(words, K):
+    """int32 words [B, 8K] -> int64 states [B, 256]: state t = the 16 stream bits that end at bit (t + 1) K - 1,
+    circular, MSB first (htr/wire.py:46-63).  Built from a doubled bit string instead of a 16-way gather."""
+    B = words.shape[0]
+    sh = torch.arange(31, -1, -1, device=words.device)
+    bits = ((words.long()[:, :, None] >> sh) & 1).reshape(B, 256 * K)
+    ext = torch.cat([bits[:, -16:], bits], 1)                      # position p of `bits` sits at p + 16
+    pw = 1 << torch.arange(15, -1, -1, device=words.device)
+    win = ext.unfold(1, 16, 1)                                      # window i covers bits i - 16 .. i - 1
+    idx = (torch.arange(256, device=words.device) + 1) * K          # window that ends at bit (t + 1) K - 1
+    return (win[:, idx, :] * pw).sum(-1)
+
+
+def dequant_Q(qweight, scales):
+    """Rotated-domain Q [m, n] float32 on the tensors' device, with torch (htr/wire.py:95-102).  Slow; the library's
+    htr_dequant_q is the fast one."""
+    mt, nt, W = qweight.shape
+    st = unpack_states(qweight.reshape(-1, W), W // 8)
+    R = codebook_f32(qweight.device)[st].reshape(mt, nt, 16, 16).permute(0, 2, 1, 3).reshape(mt * 16, nt * 16)
+    return R * scales.float()[:, None]
+
+
+def dequant(qweight, scales, su8, sv8):
+    """Original-basis W [m, n] float32 = Sv . Ho . Q . Hi . Su with torch, in the reference's order of operations
+    (htr/wire.py:105-113)."""
+    Q = dequant_Q(qweight, scales)
+    m, n = Q.shape
+    su = unpack_signs(su8, n).to(Q.device)
+    sv = unpack_signs(sv8, m).to(Q.device)
+    W = blk_had_cols_T(Q.T.contiguous()).T
+    W = blk_had_cols_T(W.contiguous())
+    return (W * sv[:, None] * su[None, :]).contiguous()
+
+
 def pack_signs(s):
     """+-1 vector [N] (N % 8 == 0) -> uint8 [N/8]; bit j%8 (LSB first) of byte j/8 set means -1 (htr/wire.py:66-69)."""
     neg = (s < 0).to(torch.int32).view(-1, 8)

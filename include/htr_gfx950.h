@@ -133,6 +133,19 @@ int htr_linear_grouped(const htr_group_entry* entries_device, int count, int m, 
 void htr_set_spin_limit(int polls);
 
 /*
+ * Encoder search: tail-biting bitshift-trellis Viterbi over the 65536 codec states, one 256-weight tile per row.
+ *   x, w      float32 [tiles, T] targets and per-element weights (T <= 256; the codec uses 256)
+ *   states    uint16 [tiles, T]: s_t with s_t >> K == s_{t-1} & (2^(16-K) - 1), circular when tailbite != 0
+ *   workspace htr_viterbi_workspace_bytes() bytes of device scratch (backpointers; no zero requirement)
+ * K = 2..7.  Same result as the reference's portable search, htr.reference.viterbi(x, w, codebook_f32(), K)
+ * (htr/reference.py:6-50), which its CUDA versions htr/vit_v1.py:46-110 and htr/vit_v2.py:100-162 also reproduce;
+ * the state values are the procedural codebook, so no codebook tensor is passed.
+ */
+size_t htr_viterbi_workspace_bytes(int64_t tiles, int T, int K);
+int htr_viterbi(const void* x, const void* w, int64_t tiles, int T, int K, int tailbite, void* states_u16,
+                void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Integer decode, tile order: out[tile, t] = v(s_t) as int16, tile = ti*(n/16)+tj, t = 16r+c.
  * Reference: decode_raw (htr/csrc/htr_kernels.cu:943-951, kernel :154-172).
  */

@@ -37,6 +37,8 @@ def parse():
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying HIP graphs")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="budget of the CPU baseline sample (0 = skip)")
     ap.add_argument("--shapes", action="store_true", help="also time every unfused shape on its own")
+    ap.add_argument("--viterbi-tiles", type=int, default=0,
+                    help="also time the encoder's trellis search on this many 256-weight tiles per K (0 = skip)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy, so a counter profile of this command holds a kernel of known traffic")
     return ap.parse_args()
@@ -207,6 +209,30 @@ def main():
                "sample": f"{reps} x (4096x4096 K4 decode to float32 W + x@W^T, batch 1) in {el:.1f} s; "
                          f"host reports {os.cpu_count()} cpus", "ms_per_matrix": round(el / reps * 1e3, 2)}
 
+    # ---- optional: the encoder's tail-biting Viterbi (htr_viterbi), tiles per second per K, with the CPU oracle beside it
+    search = None
+    if args.viterbi_tiles > 0:
+        from htr_amd import encode
+        search = {}
+        for k in (2, 3, 4, 5):
+            g = torch.Generator().manual_seed(k)
+            xv = torch.randn(args.viterbi_tiles, 256, generator=g)
+            wv = torch.rand(args.viterbi_tiles, 256, generator=g) + 0.5
+            xd, wd = xv.to(dev), wv.to(dev)
+            encode.viterbi(xd[:32], wd[:32], None, k)
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            encode.viterbi(xd, wd, None, k)
+            torch.cuda.synchronize()
+            el = time.perf_counter() - t
+            search[f"K{k}"] = {"tiles": args.viterbi_tiles, "ms": round(el * 1e3, 2), "tiles_per_s": round(args.viterbi_tiles / el)}
+            if args.cpu_seconds > 0:
+                from oracle import oracle
+                nt = 16
+                t = time.perf_counter()
+                oracle.c_viterbi(xv[:nt].numpy(), wv[:nt].numpy(), k)
+                search[f"K{k}"]["cpu_port_tiles_per_s"] = round(nt / (time.perf_counter() - t), 1)
+
     out = {
         "metric": "K4 GEMV packed-weight GB/s at batch 1 (% of 8 TB/s HBM); us per 9B decoder layer",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -224,6 +250,8 @@ def main():
     }
     if shapes is not None:
         out["shapes"] = shapes
+    if search is not None:
+        out["encoder_search"] = search
     print(json.dumps(out))
 
 

@@ -39,6 +39,9 @@ def parse():
     ap.add_argument("--shapes", action="store_true", help="also time every unfused shape on its own")
     ap.add_argument("--viterbi-tiles", type=int, default=0,
                     help="also time the encoder's trellis search on this many 256-weight tiles per K (0 = skip)")
+    ap.add_argument("--suite", nargs="*", default=None, metavar="CASE",
+                    help="also time the other baseline configurations (htr_amd/bench_suite.py): table, batch, lm_head, moe, "
+                         "prefill; no names = all")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy, so a counter profile of this command holds a kernel of known traffic")
     return ap.parse_args()
@@ -233,6 +236,13 @@ def main():
                 oracle.c_viterbi(xv[:nt].numpy(), wv[:nt].numpy(), k)
                 search[f"K{k}"]["cpu_port_tiles_per_s"] = round(nt / (time.perf_counter() - t), 1)
 
+    suite = None
+    if args.suite is not None:
+        from htr_amd import bench_suite
+        del layers, gate_up
+        torch.cuda.empty_cache()
+        suite = bench_suite.run(args.suite, dev)
+
     out = {
         "metric": "K4 GEMV packed-weight GB/s at batch 1 (% of 8 TB/s HBM); us per 9B decoder layer",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -252,6 +262,8 @@ def main():
         out["shapes"] = shapes
     if search is not None:
         out["encoder_search"] = search
+    if suite is not None:
+        out["suite"] = suite
     print(json.dumps(out))
 
 

@@ -327,8 +327,34 @@ __global__ __launch_bounds__(WG_THREADS) void k_rotate(const void* __restrict__ 
     va = load_elem(x, x_dtype, row + col + lane) * sign_of(su, col + lane);
     vb = load_elem(x, x_dtype, row + col + lane + 64) * sign_of(su, col + lane + 64);
   }
+  // max|x| of the row.  |values| compare like their bit patterns, so the scan is integer: 16 bytes per thread and load
+  // through a descriptor over the row (pieces beyond its end read zeros), four loads in flight per thread.  Rows that
+  // are not 16-byte aligned take the element-wise loop.
   float mx = 0.f;
-  for (int i = threadIdx.x; i < n; i += WG_THREADS) mx = fmaxf(mx, fabsf(load_elem(x, x_dtype, row + i)));
+  const int es = x_dtype == HTR_F32 ? 4 : 2;
+  const unsigned char* xrow = (const unsigned char*)x + row * es;
+  if ((((size_t)xrow) & 15) == 0) {
+    const __amdgpu_buffer_rsrc_t rrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)xrow, 0, n * es, 0x00020000);
+    uint32_t m32 = 0u;          // float32: max of the sign-cleared words; 16-bit types: max of the sign-cleared halves
+    for (int base = threadIdx.x * 16; base < n * es; base += 4 * WG_THREADS * 16) {
+      u4 v[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) v[u] = __builtin_amdgcn_raw_buffer_load_b128(rrsrc, base + u * WG_THREADS * 16, 0, 0);
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const uint32_t d[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          if (x_dtype == HTR_F32) m32 = max(m32, d[k] & 0x7FFFFFFFu);
+          else m32 = max(m32, max(d[k] & 0x7FFFu, (d[k] >> 16) & 0x7FFFu));
+        }
+      }
+    }
+    mx = x_dtype == HTR_F32 ? __uint_as_float(m32) : x_dtype == HTR_BF16 ? bf16_bits_to_float((uint16_t)m32) : f16_bits_to_float((uint16_t)m32);
+    if (mx != mx) mx = __uint_as_float(0x7F800000u);   // a NaN anywhere: treat the row as unbounded (scale 1)
+  } else {
+    for (int i = threadIdx.x; i < n; i += WG_THREADS) mx = fmaxf(mx, fabsf(load_elem(x, x_dtype, row + i)));
+  }
   mx = wave_max(mx);
   if (lane == 0) s_max[w] = mx;
   __syncthreads();

@@ -37,6 +37,9 @@ def viterbi(x, w, cb=None, K=4, tailbite=True):
         raise RuntimeError(f"viterbi: unsupported K {K} (2..7)")
     out = torch.empty((B, T), dtype=torch.int16, device=x.device)
     batch = max(1, min(B, MAX_SCRATCH_BYTES // per_tile))
+    cus = torch.cuda.get_device_properties(x.device).multi_processor_count
+    if B > batch >= cus:
+        batch -= batch % cus        # one workgroup per tile: whole rounds over the CUs, no launch with a few stragglers
     with torch.cuda.device(x.device):
         stream = torch.cuda.current_stream(x.device)
         need = L.htr_viterbi_workspace_bytes(batch, T, K)

@@ -22,8 +22,9 @@ NSPLIT = int(os.environ.get("HTR_NSPLIT", "0"))
 # Above this many activation rows the weight is dequantized once to the original basis (bf16) and a library GEMM does
 # the product, as the reference does for prefill (HTR_PREFILL="w", htr/ops.py:52-54,89-93); up to it, the fused
 # decode kernel runs in launches of LAUNCH_MAX_M rows (the reference's HTR_GEMV_LOOP_MAX, htr/ops.py:59-61).
-# Measured on MI355X (K4, 4096x4096 .. 14336x4096): 32-row fused launches beat dequantize + GEMM up to about 128 rows.
-GEMV_LOOP_MAX = int(os.environ.get("HTR_GEMV_LOOP_MAX", "128"))
+# Measured on MI355X (K4, eager calls): 32-row fused launches beat dequantize + GEMM up to 40 rows on 4096x4096 and up to
+# about 75 rows on 14336x4096 and 4096x14336.
+GEMV_LOOP_MAX = int(os.environ.get("HTR_GEMV_LOOP_MAX", "64"))
 
 _WORKSPACES = {}
 

@@ -162,6 +162,7 @@ int htr_dequant_q(const void* qweight, const void* scales, void* out_f32, int mt
  * Original-basis W[m, n] = Sv . Ho . Q . Hi . Su as bfloat16, row-major: the prefill path dequantizes once and hands W
  * to a library GEMM.  Reference: dequant_w (htr/csrc/htr_kernels.cu:1082-1095, kernels :657-903), used by
  * _linear_impl for M above the GEMV range (htr/ops.py:89-93); CPU definition wire.dequant (htr/wire.py:105-113).
+ * out_bf16 and sv must be 4-byte aligned (bf16 pairs are stored, the sv bits of a row block are read as words).
  */
 int htr_dequant_w(const void* qweight, const void* scales, const void* su, const void* sv, void* out_bf16,
                   int m, int n, int K, void* stream);

@@ -119,9 +119,10 @@ def test_linear_f32_out_within_tolerance(dev, oracle, K, M, shape):
 
 
 @pytest.mark.parametrize("K,M", [(3, 16), (4, 9), (4, 16), (4, 32), (3, 32), (5, 17), (4, 45), (4, 100), (2, 8), (8, 24)])
-def test_linear_small_batch_blocks(dev, oracle, K, M):
+def test_linear_small_batch_blocks(dev, oracle, K, M, monkeypatch):
     from htr_amd import ops
     print(f"linear batch K={K} M={M}", flush=True)
+    monkeypatch.setattr(ops, "GEMV_LOOP_MAX", 1 << 30)     # the fused launches at every M, also past the prefill switch
     qw, sc, su, sv, x = _case(512, 1024, K, M, 31 * K + M)
     y = ops.linear_f32out(x.to(dev), qw.to(dev), sc.to(dev), su.to(dev), sv.to(dev)).cpu().numpy()
     ref = _ref(oracle, qw, sc, su, sv, x)

@@ -30,19 +30,24 @@ _WORKSPACES = {}
 
 
 def workspace(device, stream_id, nbytes):
-    """Zeroed scratch for split partials and arrival counters, one per (device, stream).
+    """Zeroed scratch for split partials and pre-rotated activations, one per (device, stream).
 
     The reference keeps one counter tensor per device (htr/ops.py:24-28), which two streams
     would corrupt; keying by stream keeps concurrent streams apart.  Kernels leave the
-    counter words zero, so the buffer is zeroed only when it is (re)allocated.
+    partial slots zero, so the buffer is zeroed only when it is (re)allocated.
+    Calls recorded into a HIP graph use one more buffer per device, shared by every capture (a capture runs on a
+    stream of its own, and replays of one device's graphs are not expected to overlap).  Every eager call makes sure
+    that buffer exists and is large enough for its own shape, so that a capture that follows a warm-up pass over the
+    same shapes allocates nothing and records no fill.
     """
-    key = (device.index, stream_id)
-    ws = _WORKSPACES.get(key)
-    if ws is None or ws.numel() < nbytes:
-        size = max(int(nbytes), 1 << 20)
-        ws = torch.zeros(size, dtype=torch.uint8, device=device)
-        _WORKSPACES[key] = ws
-    return ws
+    capturing = torch.cuda.is_current_stream_capturing()
+    keys = [(device.index, "capture")] if capturing else [(device.index, stream_id), (device.index, "capture")]
+    for key in keys:
+        ws = _WORKSPACES.get(key)
+        if ws is None or ws.numel() < nbytes:
+            size = max(int(nbytes), 1 << 20)
+            _WORKSPACES[key] = torch.zeros(size, dtype=torch.uint8, device=device)
+    return _WORKSPACES[keys[0]]
 
 
 def _launch(x2, qweight, scales, su, sv, bias, y, m, n, K, out_code):

@@ -1,0 +1,94 @@
+"""GPU tests of how callers drive the packed linear: HIP-graph capture and replay, tracing through the registered
+custom op, and activation pointers that are only 2-byte aligned (which take the separate rotation launch)."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+REL_TOL = 1e-3
+
+
+@pytest.fixture(scope="module")
+def dev():
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    from htr_amd import _native
+    _native.lib()
+    return torch.device("cuda:0")
+
+
+def _case(m, n, K, M, seed, dtype=torch.bfloat16):
+    from htr_amd import wire
+    qw, sc, su, sv = wire.synth_linear(m, n, K, seed)
+    return qw, sc, su, sv, wire.synth_activation(M, n, seed + 7, dtype)
+
+
+def _ref(oracle, qw, sc, su, sv, x):
+    return oracle.c_linear(x.float().numpy(), qw.numpy(), sc.numpy(), su.numpy(), sv.numpy(), None)
+
+
+@pytest.mark.parametrize("M", [1, 4, 8, 40])
+def test_graph_replays_match_eager(dev, M):
+    """One captured call, replayed with new inputs, with eager launches of other shapes between the replays (they share
+    the cached workspace): every replay must give what the eager call gives, bit for bit."""
+    from htr_amd import ops, wire
+    print(f"graph replay M={M}", flush=True)
+    qw, sc, su, sv, x = _case(1024, 2048, 4, M, 4100 + M)
+    d = [t.to(dev) for t in (qw, sc, su, sv)]
+    other = [t.to(dev) for t in wire.synth_linear(2048, 1024, 3, 99)]
+    x_other = wire.synth_activation(2, 1024, 5).to(dev)
+    x_in = x.to(dev).clone()
+    ops.linear(x_in, *d)                       # warm-up: workspace allocation happens outside the capture
+    ops.linear(x_other, *other)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        y_out = ops.linear(x_in, *d)
+    for i in range(4):
+        xi = wire.synth_activation(M, 2048, 700 + i).to(dev)
+        x_in.copy_(xi)
+        ops.linear(x_other, *other)            # eager work between the replays
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        got = y_out.clone()
+        want = ops.linear(xi, *d)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), f"replay {i}"
+
+
+def test_custom_op_traces_and_runs(dev, oracle):
+    """htr::linear inside a traced function (fake-tensor shape propagation through the registered fake), run on the GPU."""
+    from htr_amd import ops
+    print("custom op under torch.compile(backend=eager)", flush=True)
+    qw, sc, su, sv, x = _case(512, 256, 4, 3, 4200)
+    d = [t.to(dev) for t in (qw, sc, su, sv)]
+
+    def f(a):
+        return torch.ops.htr.linear(a, d[0], d[1], d[2], d[3], None).float() * 2.0
+
+    fc = torch.compile(f, backend="eager", fullgraph=True)
+    y = fc(x.to(dev))
+    assert tuple(y.shape) == (3, 512)
+    assert torch.equal(y, f(x.to(dev)))
+    ref = 2.0 * _ref(oracle, qw, sc, su, sv, x)
+    assert float(np.abs(y.cpu().numpy() - ref).max() / np.abs(ref).max()) <= 2.0 ** -7      # bf16 output
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("M", [1, 3, 9])
+def test_two_byte_aligned_activations(dev, oracle, dtype, M):
+    """x that starts one element into its allocation: only 2-byte aligned, so the in-kernel rotation (dword loads) does
+    not apply and the library rotates with its own launch."""
+    from htr_amd import ops
+    print(f"2-byte aligned x dtype={dtype} M={M}", flush=True)
+    qw, sc, su, sv, x = _case(384, 512, 4, M, 4300 + M, dtype)
+    d = [t.to(dev) for t in (qw, sc, su, sv)]
+    buf = torch.zeros(M * 512 + 1, dtype=dtype, device=dev)
+    buf[1:].copy_(x.reshape(-1).to(dev))
+    xv = buf[1:].view(M, 512)
+    assert xv.data_ptr() % 4 == 2 and xv.is_contiguous()
+    y = ops.linear_f32out(xv, *d).cpu().numpy()
+    ref = _ref(oracle, qw, sc, su, sv, x)
+    assert float(np.abs(y - ref).max() / np.abs(ref).max()) <= REL_TOL

@@ -92,3 +92,45 @@ def test_two_byte_aligned_activations(dev, oracle, dtype, M):
     y = ops.linear_f32out(xv, *d).cpu().numpy()
     ref = _ref(oracle, qw, sc, su, sv, x)
     assert float(np.abs(y - ref).max() / np.abs(ref).max()) <= REL_TOL
+
+
+def test_encode_save_load_plugin_apply(dev, tmp_path):
+    """The whole chain on the device: encode two projections over one input with a shared sign vector (GPU search),
+    save them as a checkpoint, read it back, place the shards through the plugin's weight loaders into one fused
+    module, and run the module: the result is x times the encoder's own reconstruction of the weights."""
+    from htr_amd import checkpoint, encode, vllm_plugin as vp
+    print("encode -> checkpoint -> plugin loaders -> apply", flush=True)
+
+    class _Linear(vp.LinearBase):
+        pass
+
+    g = torch.Generator().manual_seed(77)
+    Wg, Wu = torch.randn(256, 256, generator=g) * 0.03, torch.randn(128, 256, generator=g) * 0.03
+    A = torch.randn(512, 256, generator=g)
+    H = (A.T @ A / 512).to(dev)
+    res = encode.encode_group([{"W": Wg.to(dev), "H": H}, {"W": Wu.to(dev), "H": H}], 4, seed=5, shared_su=True, max_batch=4096)
+    path = str(tmp_path / "model.safetensors")
+    checkpoint.save_linears(path, {"model.layers.0.mlp.gate_proj": tuple(res[0][k] for k in ("qweight", "scales", "su", "sv")),
+                                   "model.layers.0.mlp.up_proj": tuple(res[1][k] for k in ("qweight", "scales", "su", "sv"))})
+    ck = checkpoint.Checkpoint(path)
+    layer = _Linear()
+    meth = vp.HTRLinearMethod(4)
+    meth.create_weights(layer, 256, [256, 128], 256, 384, torch.bfloat16)
+    for sid, name in enumerate(("gate_proj", "up_proj")):
+        qw, sc, su, sv = ck.linear(f"model.layers.0.mlp.{name}")
+        layer.htr_qweight.weight_loader(layer.htr_qweight, qw, sid)
+        layer.htr_scales.weight_loader(layer.htr_scales, sc, sid)
+        layer.htr_su.weight_loader(layer.htr_su, su, sid)
+        layer.htr_sv.weight_loader(layer.htr_sv, sv, sid)
+    for nm in ("htr_qweight", "htr_scales", "htr_su", "htr_sv"):
+        getattr(layer, nm).data = getattr(layer, nm).data.to(dev)
+    meth.process_weights_after_loading(layer)
+    x = torch.randn(5, 256, generator=g).bfloat16()
+    y = meth.apply(layer, x.to(dev)).float().cpu()
+    What = torch.cat([res[0]["What"], res[1]["What"]]).float().cpu()
+    ref = x.float() @ What.T
+    assert tuple(y.shape) == (5, 384)
+    assert float((y - ref).abs().max() / ref.abs().max()) <= 2.0 ** -7          # bf16 output
+    # and the encoding is a faithful one: within a few percent of the dense product
+    dense = x.float() @ torch.cat([Wg, Wu]).T
+    assert float((ref - dense).norm() / dense.norm()) < 0.2

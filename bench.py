@@ -170,6 +170,19 @@ def main():
                 "kernel": "k_linear<K=4,MB=1> 28672x4096 (gate_up) batch 1", "us_per_launch": round(dom_us, 3),
                 "algorithmic_bytes_per_launch": dom_bytes}
 
+    # co-bound: the rate at which the SIMDs issue the decode's integer instructions.  Wave instructions per launch come
+    # from the committed counter profile, the duration is the one measured above; peak = 256 CUs x 4 SIMDs x 16 lanes
+    # per cycle at the 2.4 GHz peak engine clock.
+    cpath = os.path.join(ROOT, "profiles", "k_linear_K4_gate_up_sq_counters.json")
+    if os.path.exists(cpath):
+        with open(cpath) as f:
+            cj = json.load(f)
+        lane_ops = (cj["valu_instructions_per_launch"] + cj["mfma_instructions_per_launch"]) * 64
+        peak = 256 * 4 * 16 * 2.4e9 / 1e12
+        roofline["co_bound"] = {"kind": "valu_issue", "unit": "T lane-ops/s", "achieved": round(lane_ops / dom_us / 1e6, 2),
+                                "peak": round(peak, 2), "frac": round(lane_ops / dom_us / 1e6 / peak, 4),
+                                "valu_instructions_per_weight": round(cj["valu_instructions_per_launch"] * 64 / cj["weights_per_launch"], 3)}
+
     if args.calibrate_copy:
         src = torch.randint(0, 256, (256 << 20,), dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)

@@ -1517,14 +1517,19 @@ inline bool make_batch_plan(int m, int n, int M, int want_S, BatchPlan& bp) {
   // Measured on MI355X (K4, 8..32 rows, 4096..28672 output rows): one workgroup per CU is the best fill; every further
   // split adds partial traffic that grows with the rows.  So: the largest split that keeps the grid within the CU
   // count, among the splits that leave no column range empty.
+  // Splits shorter than 8 column blocks cost more in partial traffic and set-up than their parallelism returns
+  // (4096x4096, 16 and 32 rows: 4 splits of 8 blocks beat 8 of 4 by 5..8 %), unless fewer than half the CUs would have work.
   const int limit = want_S > 0 ? want_S : (NUM_CU / rbs > 1 ? NUM_CU / rbs : 1);
-  bool found = false;
+  bool found = false, found_long = false;
+  BatchPlan longer = bp;
   for (int S = 1; S <= nblk && S <= limit; ++S) {
     const int cb = (nblk + S - 1) / S;
     if ((nblk + cb - 1) / cb != S) continue;                       // some split would be empty
     if (want_S > 0 && S != want_S) continue;
     bp.S = S; bp.cb = cb; bp.wgs = rbs * S; found = true;
+    if (cb >= 8 && rbs * S >= NUM_CU / 2) { longer = bp; found_long = true; }
   }
+  if (want_S <= 0 && found_long && M > 8) bp = longer;           // with 8 rows the partials are small: keep the fill
   return found;
 }
 

@@ -220,10 +220,21 @@ def main():
             el = time.perf_counter() - t
             if el >= args.cpu_seconds or reps >= 200:
                 break
+        # second shape of the same baseline: the factorised product (rotate x, decode rows on the fly, rotate y; float64),
+        # which never materialises W
+        oracle.c_linear(x, *a)
+        freps, ft = 0, time.perf_counter()
+        while True:
+            oracle.c_linear(x, *a)
+            freps += 1
+            fel = time.perf_counter() - ft
+            if fel >= args.cpu_seconds / 3 or freps >= 100:
+                break
         b = wire.payload_bytes(m, n, K)
         cpu = {"value": round(b * reps / el / 1e9, 4), "unit": "GB/s", "cores": oracle.c_num_threads(), "kind": "port",
                "sample": f"{reps} x (4096x4096 K4 decode to float32 W + x@W^T, batch 1) in {el:.1f} s; "
-                         f"host reports {os.cpu_count()} cpus", "ms_per_matrix": round(el / reps * 1e3, 2)}
+                         f"host reports {os.cpu_count()} cpus", "ms_per_matrix": round(el / reps * 1e3, 2),
+               "fused_decode_gemv_value": round(b * freps / fel / 1e9, 4), "fused_decode_gemv_ms_per_matrix": round(fel / freps * 1e3, 2)}
 
     # ---- optional: the encoder's tail-biting Viterbi (htr_viterbi), tiles per second per K, with the CPU oracle beside it
     search = None

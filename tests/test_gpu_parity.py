@@ -184,6 +184,30 @@ def test_large_activations_do_not_overflow(dev, oracle):
         assert _rel(y[r], ref[r]) <= REL_TOL
 
 
+@pytest.mark.parametrize("M", [1, 3, 9])
+def test_zero_tiny_and_non_finite_activations(dev, oracle, M):
+    """All-zero rows give exactly the bias, rows of 1e-30 keep their relative accuracy, and an infinity or a NaN in a
+    row stays in that row (every output of it non-finite) without touching the other rows."""
+    from htr_amd import ops
+    print(f"linear zero / tiny / inf rows M={M}", flush=True)
+    qw, sc, su, sv, x = _case(256, 384, 4, M, 123 + M, torch.float32)
+    d = [t.to(dev) for t in (qw, sc, su, sv)]
+    bias = torch.randn(256, generator=torch.Generator().manual_seed(3))
+    z = ops.linear_f32out(torch.zeros_like(x).to(dev), *d, bias.to(dev)).cpu()
+    assert torch.equal(z, bias.expand(M, 256))
+    tiny = x * 1e-30
+    y = ops.linear_f32out(tiny.to(dev), *d).cpu().numpy()
+    assert _rel(y, _ref(oracle, qw, sc, su, sv, tiny)) <= REL_TOL
+    for bad in (float("inf"), float("nan")):
+        xb = x.clone()
+        xb[M - 1, 17] = bad
+        yb = ops.linear_f32out(xb.to(dev), *d).cpu().numpy()
+        assert not np.any(np.isfinite(yb[M - 1]))
+        if M > 1:
+            ref = _ref(oracle, qw, sc, su, sv, x)
+            assert _rel(yb[:M - 1], ref[:M - 1]) <= REL_TOL
+
+
 def test_zero_rows_and_repeatability(dev):
     from htr_amd import ops
     print("linear M=0 / repeat", flush=True)

@@ -113,3 +113,22 @@ def save_linears(path, linears, metadata=None):
         for suf, v in zip(SUFFIXES, t):
             flat[f"{prefix}.{suf}"] = v.detach().cpu().clone().contiguous()      # own storage: parts of a fused module share su
     save_file(flat, path, metadata={"format": "pt", **(metadata or {})})
+
+
+def quantization_config(linears):
+    """The `quantization_config` entry of config.json for {prefix: (qweight, scales, su, sv)}, as the reference's
+    converter writes it (htr/quantize.py:282-283): wire, generator and geometry constants plus the bit width per module."""
+    return {"quant_method": "htr", **_EXPECT,
+            "modules": {prefix: {"K": wire.check_shapes(*t)[2]} for prefix, t in linears.items()}}
+
+
+def save_checkpoint(directory, linears, config=None):
+    """A checkpoint directory `Checkpoint` (and the plugin's HTRConfig.from_config) can read: model.safetensors with the
+    packed tensors and config.json = `config` (a dict, e.g. the dense model's) with the HTR table put in."""
+    os.makedirs(directory, exist_ok=True)
+    save_linears(os.path.join(directory, "model.safetensors"), linears)
+    cfg = dict(config or {})
+    cfg["quantization_config"] = quantization_config(linears)
+    with open(os.path.join(directory, "config.json"), "w") as f:
+        json.dump(cfg, f, indent=2)
+    return cfg

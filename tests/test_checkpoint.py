@@ -67,3 +67,18 @@ def test_config_validation(tmp_path):
     json.dump(cfg, open(tmp_path / "config.json", "w"))
     with pytest.raises(ValueError):
         checkpoint.Checkpoint(str(tmp_path)).linear("model.layers.0.self_attn.o_proj")
+
+
+def test_save_checkpoint_writes_what_the_reader_and_the_plugin_expect(tmp_path):
+    from htr_amd import vllm_plugin as vp
+    lin = {"model.layers.0.mlp.gate_proj": wire.synth_linear(256, 128, 3, 1), "lm_head": wire.synth_linear(128, 128, 5, 2)}
+    cfg = checkpoint.save_checkpoint(str(tmp_path / "ck"), lin, {"architectures": ["X"]})
+    qc = cfg["quantization_config"]
+    assert qc["quant_method"] == "htr" and qc["wire"] == "HTR-W1" and qc["generator"] == "rdna24"
+    assert (qc["L"], qc["tile"], qc["rht_block"]) == (16, 16, 128) and cfg["architectures"] == ["X"]
+    ck = checkpoint.Checkpoint(str(tmp_path / "ck"))
+    assert ck.modules == {"model.layers.0.mlp.gate_proj": 3, "lm_head": 5}
+    for p, want in lin.items():
+        assert all(torch.equal(a, b) for a, b in zip(ck.linear(p), want))
+    hc = vp.HTRConfig.from_config(qc)
+    assert hc.modules == {"layers.0.mlp.gate_proj": 3, "lm_head": 5}

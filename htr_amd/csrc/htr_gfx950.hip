@@ -478,6 +478,9 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
     const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)x, 0, M * n * 2, 0x00020000);
     const __amdgpu_buffer_rsrc_t srsrc = __builtin_amdgcn_make_buffer_rsrc((void*)su, 0, n >> 3, 0x00020000);
     constexpr int OUT_OF_RANGE = 0x7FFFFF00;
+    // every offset first, then the loads back to back: with address arithmetic (and its branches) between two loads
+    // the compiler waits for the first load to return before it issues the second one and the weight stream behind it
+    int xoff[NPW], soff[NPW];
 #pragma unroll
     for (int tt = 0; tt < NPW; ++tt) {
       const int pi = w + tt * WG_WAVES;
@@ -485,19 +488,33 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
       prow[tt] = M == 1 ? 0 : pi / nbl;
       pli[tt] = pi - prow[tt] * nbl;
       const int col = pair_col(pli[tt]);
-      xr[tt] = __builtin_amdgcn_raw_buffer_load_b32(xrsrc, live ? (prow[tt] * n + col) * 2 + 4 * lane : OUT_OF_RANGE, 0, 0);
-      sb[tt] = (uint32_t)(uint8_t)__builtin_amdgcn_raw_buffer_load_b8(srsrc, live ? (col >> 3) + (lane >> 2) : OUT_OF_RANGE, 0, 0);
+      xoff[tt] = live ? (prow[tt] * n + col) * 2 + 4 * lane : OUT_OF_RANGE;
+      soff[tt] = live ? (col >> 3) + (lane >> 2) : OUT_OF_RANGE;
     }
+    HTR_PIN();
+#pragma unroll
+    for (int tt = 0; tt < NPW; ++tt) {
+      xr[tt] = __builtin_amdgcn_raw_buffer_load_b32(xrsrc, xoff[tt], 0, 0);
+      sb[tt] = (uint32_t)(uint8_t)__builtin_amdgcn_raw_buffer_load_b8(srsrc, soff[tt], 0, 0);
+    }
+    HTR_PIN();
   } else {
-    // with pre-rotated activations: 16-byte pieces of this chunk's x~ slice
+    // with pre-rotated activations: 16-byte pieces of this chunk's x~ slice, through a descriptor over x~ so that the
+    // pieces beyond the slice need no branch; offsets first, then the loads back to back (a branch or address
+    // arithmetic between two loads makes the compiler wait for the first one before it issues anything else)
+    const __amdgpu_buffer_rsrc_t crsrc = __builtin_amdgcn_make_buffer_rsrc((void*)t.xt_g, 0, M * n * 2, 0x00020000);
+    constexpr int OUT_OF_RANGE = 0x7FFFFF00;
+    int coff[COPY_REGS];
 #pragma unroll
     for (int tt = 0; tt < COPY_REGS; ++tt) {
       const int ci = threadIdx.x + tt * WG_THREADS;
-      if (ci < ncopy) {
-        const int pi = ci >> 4, mrow = pi / nbl, li = pi - mrow * nbl;
-        cp[tt] = *(const u4*)(t.xt_g + (size_t)mrow * n + pair_col(li) + (ci & 15) * 8);
-      }
+      const int pi = ci >> 4, mrow = M == 1 ? 0 : pi / nbl, li = pi - mrow * nbl;
+      coff[tt] = ci < ncopy ? (mrow * n + pair_col(li) + (ci & 15) * 8) * 2 : OUT_OF_RANGE;
     }
+    HTR_PIN();
+#pragma unroll
+    for (int tt = 0; tt < COPY_REGS; ++tt) cp[tt] = __builtin_amdgcn_raw_buffer_load_b128(crsrc, coff[tt], 0, 0);
+    HTR_PIN();
   }
 
   // ---- the weight stream.  This wave's strip of row block rb is tile row rb * 8 + w; its 8 tiles of column block blk

@@ -68,6 +68,22 @@ __device__ __forceinline__ void store_elem(void* p, int dtype, size_t idx, float
   else if (dtype == HTR_F16) ((uint16_t*)p)[idx] = __builtin_bit_cast(uint16_t, (_Float16)v);
   else ((float*)p)[idx] = v;
 }
+// The same through pointers that are known to be global memory (kernel-argument structs lose that, and generic
+// accesses compile to flat instructions, which also count against the LDS counter)
+#define HTR_GLOBAL __attribute__((address_space(1)))
+__device__ __forceinline__ float load_elem_g(const void* p, int dtype, size_t idx) {
+  if (dtype == HTR_BF16) return bf16_bits_to_float(((const HTR_GLOBAL uint16_t*)p)[idx]);
+  if (dtype == HTR_F16) return f16_bits_to_float(((const HTR_GLOBAL uint16_t*)p)[idx]);
+  return ((const HTR_GLOBAL float*)p)[idx];
+}
+__device__ __forceinline__ void store_elem_g(void* p, int dtype, size_t idx, float v) {
+  if (dtype == HTR_BF16) ((HTR_GLOBAL uint16_t*)p)[idx] = float_to_bf16_bits(v);
+  else if (dtype == HTR_F16) ((HTR_GLOBAL uint16_t*)p)[idx] = __builtin_bit_cast(uint16_t, (_Float16)v);
+  else ((HTR_GLOBAL float*)p)[idx] = v;
+}
+__device__ __forceinline__ float sign_of_g(const uint8_t* bits, int j) {
+  return ((((const HTR_GLOBAL uint8_t*)bits)[j >> 3] >> (j & 7)) & 1) ? -1.f : 1.f;
+}
 __device__ __forceinline__ float sign_of(const uint8_t* bits, int j) { return ((bits[j >> 3] >> (j & 7)) & 1) ? -1.f : 1.f; }
 // ---- cross-lane exchange without LDS round trips: DPP for lane xor 1, 2, 4, 8; gfx950 row swaps for 16 and 32
 template <int CTRL> __device__ __forceinline__ float dpp_mov(float v) {
@@ -462,6 +478,10 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
   float* s_fin = (float*)(lds + lds_fin_offset(M, nblmax));
 
   const int npairs = M * nbl;
+  // pair index -> activation row: pi / nbl for pi < 2^16 through the float reciprocal (the quotient's fraction is at
+  // least 0.5 / nbl away from an integer, far more than the rounding error), instead of an integer division per use
+  const float inv_nbl = 1.0f / (float)nbl;
+  auto row_of_pair = [&](int pi) { return M == 1 ? 0 : (int)(((float)pi + 0.5f) * inv_nbl); };
   auto pair_col = [&](int li) { int b = all_blocks ? li : c0 + li; if (b >= nblk) b -= nblk; return b * 128; };
 
   // ---- activations first: they head the longest dependency chain.  Wave w rotates the (row, block) pairs w and w + 8:
@@ -473,6 +493,7 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
   int prow[NPW], pli[NPW];
   constexpr int COPY_REGS = 4;
   u4 cp[COPY_REGS];
+  int cdst[COPY_REGS];
   const int ncopy = npairs * 16;                 // 16 pieces of 8 halves per (row, block) pair
   if constexpr (!PREROT) {
     const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)x, 0, M * n * 2, 0x00020000);
@@ -485,7 +506,7 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
     for (int tt = 0; tt < NPW; ++tt) {
       const int pi = w + tt * WG_WAVES;
       const bool live = pi < npairs;
-      prow[tt] = M == 1 ? 0 : pi / nbl;
+      prow[tt] = row_of_pair(pi);
       pli[tt] = pi - prow[tt] * nbl;
       const int col = pair_col(pli[tt]);
       xoff[tt] = live ? (prow[tt] * n + col) * 2 + 4 * lane : OUT_OF_RANGE;
@@ -508,13 +529,50 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
 #pragma unroll
     for (int tt = 0; tt < COPY_REGS; ++tt) {
       const int ci = threadIdx.x + tt * WG_THREADS;
-      const int pi = ci >> 4, mrow = M == 1 ? 0 : pi / nbl, li = pi - mrow * nbl;
+      const int pi = ci >> 4, mrow = row_of_pair(pi), li = pi - mrow * nbl;
       coff[tt] = ci < ncopy ? (mrow * n + pair_col(li) + (ci & 15) * 8) * 2 : OUT_OF_RANGE;
+      cdst[tt] = mrow * rowh + li * 128 + (ci & 1) * 64 + ((ci & 15) >> 1) * 8;      // where the piece goes in LDS
     }
     HTR_PIN();
 #pragma unroll
     for (int tt = 0; tt < COPY_REGS; ++tt) cp[tt] = __builtin_amdgcn_raw_buffer_load_b128(crsrc, coff[tt], 0, 0);
     HTR_PIN();
+  }
+
+  // row constants of a finished row block (scale, output sign, bias).  The wave's first (segment, row) pair requests
+  // them here, with the activation loads and ahead of the weight stream (loads return in order: behind the stream
+  // they would hold up the first decode), and only keeps the raw bits, which the output side converts at the end.
+  // (Only where the workgroup rotates its own activations: in the kernel for pre-rotated activations the six
+  // registers, held through the loop, would cost a wave of occupancy; there the request goes out before the last
+  // barrier.)
+  struct RowRaw { uint32_t sc0, sc1, sv0, sv1, b0, b1; };
+  auto row_load = [&](int rb, RowRaw& r) {
+    const int r0 = rb * 128 + lane, r1 = r0 + 64;
+    r.sc0 = ((const HTR_GLOBAL uint16_t*)t.scales)[r0];
+    r.sc1 = ((const HTR_GLOBAL uint16_t*)t.scales)[r1];
+    r.sv0 = ((const HTR_GLOBAL uint8_t*)t.sv)[r0 >> 3];
+    r.sv1 = ((const HTR_GLOBAL uint8_t*)t.sv)[r1 >> 3];
+    r.b0 = 0u; r.b1 = 0u;
+    if (t.bias != nullptr) {
+      if (y_dtype == HTR_F32) { r.b0 = ((const HTR_GLOBAL uint32_t*)t.bias)[r0]; r.b1 = ((const HTR_GLOBAL uint32_t*)t.bias)[r1]; }
+      else { r.b0 = ((const HTR_GLOBAL uint16_t*)t.bias)[r0]; r.b1 = ((const HTR_GLOBAL uint16_t*)t.bias)[r1]; }
+    }
+  };
+  auto row_finish = [&](const RowRaw& r, float& rs0, float& rs1, float& b0v, float& b1v) {
+    rs0 = f16_bits_to_float((uint16_t)r.sc0) * t.cbscale * INV_SQRT128;
+    rs1 = f16_bits_to_float((uint16_t)r.sc1) * t.cbscale * INV_SQRT128;
+    // output sign of rows lane and lane + 64 (bit lane % 8 of their sv bytes) folded into the scale that is applied
+    // after the rotation
+    rs0 = ((r.sv0 >> (lane & 7)) & 1u) ? -rs0 : rs0;
+    rs1 = ((r.sv1 >> (lane & 7)) & 1u) ? -rs1 : rs1;
+    auto cvt = [&](uint32_t b) {
+      return y_dtype == HTR_F32 ? __uint_as_float(b) : y_dtype == HTR_BF16 ? bf16_bits_to_float((uint16_t)b) : f16_bits_to_float((uint16_t)b);
+    };
+    b0v = cvt(r.b0); b1v = cvt(r.b1);
+  };
+  RowRaw first_raw = {0u, 0u, 0u, 0u, 0u, 0u};
+  if constexpr (!PREROT) {
+    if (w < nfin * M) row_load(rb_first + (M == 1 ? w : w / M), first_raw);
   }
 
   // ---- the weight stream.  This wave's strip of row block rb is tile row rb * 8 + w; its 8 tiles of column block blk
@@ -605,18 +663,15 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
 #pragma unroll
     for (int tt = 0; tt < COPY_REGS; ++tt) {
       const int ci = threadIdx.x + tt * WG_THREADS;
-      if (ci < ncopy) {
-        const int pi = ci >> 4, mrow = pi / nbl, li = pi - mrow * nbl;
-        *(u4*)(xt + (size_t)mrow * rowh + li * 128 + (ci & 1) * 64 + ((ci & 15) >> 1) * 8) = cp[tt];
-      }
+      if (ci < ncopy) *(u4*)(xt + cdst[tt]) = cp[tt];
     }
     for (int ci = threadIdx.x + COPY_REGS * WG_THREADS; ci < ncopy; ci += WG_THREADS) {
-      const int pi = ci >> 4, mrow = pi / nbl, li = pi - mrow * nbl;
+      const int pi = ci >> 4, mrow = row_of_pair(pi), li = pi - mrow * nbl;
       *(u4*)(xt + (size_t)mrow * rowh + li * 128 + (ci & 1) * 64 + ((ci & 15) >> 1) * 8) =
           *(const u4*)(t.xt_g + (size_t)mrow * n + pair_col(li) + (ci & 15) * 8);
     }
     for (int i = threadIdx.x; i < npairs * 2; i += WG_THREADS) {
-      const int pi = i >> 1, mrow = pi / nbl, li = pi - mrow * nbl;
+      const int pi = i >> 1, mrow = row_of_pair(pi), li = pi - mrow * nbl;
       s_xs[i] = t.xs_g[((size_t)mrow * nblk + (pair_col(li) >> 7)) * 2 + (i & 1)];
     }
   }
@@ -760,26 +815,22 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
   // ---- output side of the row blocks that end in this chunk (nfin of them): wave w takes (segment, activation row)
   // pairs w, w + 8, ...
   const size_t slot_floats = (size_t)M * 128;
-  // row constants of the wave's first pair are fetched before the barrier: they do not depend on the partials
-  auto row_consts = [&](int rb, float& rs0, float& rs1, float& b0v, float& b1v) {
-    const int r0 = rb * 128 + lane, r1 = r0 + 64;
-    rs0 = f16_bits_to_float(t.scales[r0]) * t.cbscale * INV_SQRT128;
-    rs1 = f16_bits_to_float(t.scales[r1]) * t.cbscale * INV_SQRT128;
-    b0v = 0.f; b1v = 0.f;
-    if (t.bias != nullptr) { b0v = load_elem(t.bias, y_dtype, r0); b1v = load_elem(t.bias, y_dtype, r1); }
-    // output sign of rows lane and lane + 64 folded into the scale that is applied after the rotation
-    rs0 = sign_of(t.sv, r0) < 0.f ? -rs0 : rs0;
-    rs1 = sign_of(t.sv, r1) < 0.f ? -rs1 : rs1;
-  };
-  float f_rs0 = 0.f, f_rs1 = 0.f, f_b0 = 0.f, f_b1 = 0.f;
   if (nfin == 0) return;        // a pure contributor: its partial is on its way, nothing else to do (uniform)
-  if (w < nfin * M) row_consts(rb_first + (M == 1 ? w : w / M), f_rs0, f_rs1, f_b0, f_b1);
+  if constexpr (PREROT) {
+    if (w < nfin * M) row_load(rb_first + (M == 1 ? w : w / M), first_raw);
+  }
   __syncthreads();
   for (int idx = w; idx < nfin * M; idx += WG_WAVES) {
     const int seg = M == 1 ? idx : idx / M, mrow = idx - seg * M, rb = rb_first + seg;
     const int r0 = rb * 128 + lane, r1 = r0 + 64;
-    float rs0 = f_rs0, rs1 = f_rs1, b0v = f_b0, b1v = f_b1;
-    if (idx != w) row_consts(rb, rs0, rs1, b0v, b1v);
+    float rs0, rs1, b0v, b1v;
+    if (idx == w) {
+      row_finish(first_raw, rs0, rs1, b0v, b1v);
+    } else {
+      RowRaw rr;
+      row_load(rb, rr);
+      row_finish(rr, rs0, rs1, b0v, b1v);
+    }
     float v0s = 0.f, v1s = 0.f;
     bool failed = false;
     if (seg == 0 && c0 != 0) {
@@ -829,8 +880,8 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
     v0s = __builtin_fmaf(v0s, rs0 < 0.f ? -1.f : 1.f, b0v);
     v1s = __builtin_fmaf(v1s, rs1 < 0.f ? -1.f : 1.f, b1v);
     if (failed) { v0s = __builtin_nanf(""); v1s = v0s; }
-    store_elem(t.y, y_dtype, (size_t)mrow * m + r0, v0s);
-    store_elem(t.y, y_dtype, (size_t)mrow * m + r1, v1s);
+    store_elem_g(t.y, y_dtype, (size_t)mrow * m + r0, v0s);
+    store_elem_g(t.y, y_dtype, (size_t)mrow * m + r1, v1s);
   }
 }
 
@@ -891,6 +942,22 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear_batch(const uint32_t* __r
   }
   stage_load(c_begin, 0);
   stage_load(c_begin + 1, 1);
+
+  // row constants of the output side (scale, sign, bias of rows lane and lane + 64), requested ahead of the weight stream by the workgroup
+  // that will finish the row block, so that they have long arrived when it needs them
+  const bool finisher = s_idx == S - 1;
+  const int r0 = rb * 128 + lane, r1 = r0 + 64;
+  uint32_t raw_sc0 = 0u, raw_sc1 = 0u, raw_sv0 = 0u, raw_sv1 = 0u, raw_b0 = 0u, raw_b1 = 0u;   // bits only: converted at the end
+  if (finisher) {
+    raw_sc0 = ((const HTR_GLOBAL uint16_t*)t.scales)[r0];
+    raw_sc1 = ((const HTR_GLOBAL uint16_t*)t.scales)[r1];
+    raw_sv0 = ((const HTR_GLOBAL uint8_t*)t.sv)[r0 >> 3];
+    raw_sv1 = ((const HTR_GLOBAL uint8_t*)t.sv)[r1 >> 3];
+    if (t.bias != nullptr) {
+      if (y_dtype == HTR_F32) { raw_b0 = ((const HTR_GLOBAL uint32_t*)t.bias)[r0]; raw_b1 = ((const HTR_GLOBAL uint32_t*)t.bias)[r1]; }
+      else { raw_b0 = ((const HTR_GLOBAL uint16_t*)t.bias)[r0]; raw_b1 = ((const HTR_GLOBAL uint16_t*)t.bias)[r1]; }
+    }
+  }
 
   // ---- the weight stream of this wave: one contiguous piece of its strip
   constexpr int STEP_BYTES = 256 * K;
@@ -984,7 +1051,6 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear_batch(const uint32_t* __r
   }
 
   // ---- this wave's strip partial per activation row: offset removed, activation scale undone, tile parities added
-  const bool finisher = s_idx == S - 1;
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
     const int mrow = mb * 8 + (n16 >> 1);
@@ -1015,12 +1081,13 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear_batch(const uint32_t* __r
   if (!finisher) return;
 
   // ---- output side: the last split of the row block adds the other splits' partials (fixed order) and finishes
-  const int r0 = rb * 128 + lane, r1 = r0 + 64;
-  float rs0 = f16_bits_to_float(t.scales[r0]) * t.cbscale * INV_SQRT128;
-  float rs1 = f16_bits_to_float(t.scales[r1]) * t.cbscale * INV_SQRT128;
-  const float sg0 = sign_of(t.sv, r0), sg1 = sign_of(t.sv, r1);
-  float b0v = 0.f, b1v = 0.f;
-  if (t.bias != nullptr) { b0v = load_elem(t.bias, y_dtype, r0); b1v = load_elem(t.bias, y_dtype, r1); }
+  const float rs0 = f16_bits_to_float((uint16_t)raw_sc0) * t.cbscale * INV_SQRT128;
+  const float rs1 = f16_bits_to_float((uint16_t)raw_sc1) * t.cbscale * INV_SQRT128;
+  const float sg0 = ((raw_sv0 >> (lane & 7)) & 1u) ? -1.f : 1.f, sg1 = ((raw_sv1 >> (lane & 7)) & 1u) ? -1.f : 1.f;
+  auto cvt_bias = [&](uint32_t b) {
+    return y_dtype == HTR_F32 ? __uint_as_float(b) : y_dtype == HTR_BF16 ? bf16_bits_to_float((uint16_t)b) : f16_bits_to_float((uint16_t)b);
+  };
+  const float b0v = cvt_bias(raw_b0), b1v = cvt_bias(raw_b1);
   __syncthreads();
   for (int mrow = w; mrow < M; mrow += WG_WAVES) {
     float v0s = 0.f, v1s = 0.f;
@@ -1067,8 +1134,8 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear_batch(const uint32_t* __r
     v0s = __builtin_fmaf(v0s, sg0, b0v);
     v1s = __builtin_fmaf(v1s, sg1, b1v);
     if (failed) { v0s = __builtin_nanf(""); v1s = v0s; }
-    store_elem(t.y, y_dtype, (size_t)mrow * m + r0, v0s);
-    store_elem(t.y, y_dtype, (size_t)mrow * m + r1, v1s);
+    store_elem_g(t.y, y_dtype, (size_t)mrow * m + r0, v0s);
+    store_elem_g(t.y, y_dtype, (size_t)mrow * m + r1, v1s);
   }
 }
 

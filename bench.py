@@ -1,8 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the MI355X HTR-W1 packed-linear path.  Prints ONE JSON line.
 
-Workload (BASELINE.json configs[2], which contains every shape of configs[1] at K4, batch 1): the packed
-linears of one dense 9B-class decoder layer at K4, one bf16 activation row per linear.
+Workload: the packed linears of one dense 9B-class decoder layer at K4, one bf16 activation row per linear.
 A "step" is one layer: qkv (6144x4096, q/k/v fused along the output dim as the wire format allows),
 o (4096x4096), gate_up (28672x4096, fused) and down (4096x14336): four launches through the C ABI.  Weights
 cycle through a ring of distinct layer copies (>= 1 GB) so neither the per-XCD L2 nor the 256 MB Infinity

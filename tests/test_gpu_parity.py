@@ -247,7 +247,7 @@ def test_full_size_shapes(dev, oracle, K, m, n):
     assert np.array_equal(y2, 2 * y)
 
 
-# ---- BASELINE configs 4 and 5 as parity cases
+# ---- the small-batch GEMM shapes, the 64-expert stack and the output head as parity cases
 @pytest.mark.parametrize("K,M,m,n", [(3, 8, 14336, 4096), (4, 16, 14336, 4096), (4, 32, 4096, 14336), (3, 32, 14336, 4096),
                                      (4, 8, 4096, 14336)])
 def test_small_batch_gemm_shapes(dev, oracle, K, M, m, n):
@@ -330,7 +330,7 @@ def test_grouped_launch_matches_single_launches(dev, oracle):
 
 
 def test_moe_64_experts_grouped(dev, oracle):
-    """BASELINE configuration 5, all 64 experts materialised: gate/up 1408x2048 (fused to 2816x2048) and down 2048x1408
+    """The 64-expert configuration, all experts materialised: gate/up 1408x2048 (fused to 2816x2048) and down 2048x1408
     at K4, top-6 routing of 16 tokens with seeded softmax-routed ids; two grouped launches against the per-expert
     composition on the CPU oracle."""
     from htr_amd import ops, wire

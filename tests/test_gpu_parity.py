@@ -365,3 +365,30 @@ def test_lm_head_shape(dev, oracle):
     y = ops.linear_f32out(x.to(dev), *[t.to(dev) for t in (qw, sc, su, sv)]).cpu().numpy()
     ref = _ref(oracle, qw, sc, su, sv, x)
     assert _rel(y, ref) <= REL_TOL, _rel(y, ref)
+
+
+def test_seeded_sweep_of_shapes_rows_and_widths(dev, oracle):
+    """Forty-eight seeded combinations of output and input size (multiples of 128 up to 2048, so every chunking case
+    of the planner: aligned, ragged, chunks across row blocks, a single workgroup), bit width, row count (all three
+    kernels: chunked, batched, fused-launch loop), activation type and bias, each against the float64 oracle."""
+    from htr_amd import ops
+    rng = np.random.default_rng(20261125)
+    worst = 0.0
+    for case in range(48):
+        m = int(rng.integers(1, 17)) * 128
+        n = int(rng.integers(1, 17)) * 128
+        K = int(rng.choice([2, 3, 4, 5, 6, 7, 8]))
+        M = int(rng.choice([1, 1, 1, 2, 3, 4, 5, 7, 8, 9, 15, 16, 17, 31, 32, 33, 40]))
+        dtype = [torch.bfloat16, torch.float16, torch.float32][int(rng.integers(0, 3))]
+        with_bias = bool(rng.integers(0, 2))
+        print(f"sweep case {case}: {m}x{n} K={K} M={M} {dtype} bias={with_bias}", flush=True)
+        qw, sc, su, sv, x = _case(m, n, K, M, 9000 + case, dtype)
+        bias = torch.randn(m, generator=torch.Generator().manual_seed(case)) if with_bias else None
+        y = ops.linear_f32out(x.to(dev), qw.to(dev), sc.to(dev), su.to(dev), sv.to(dev),
+                              None if bias is None else bias.to(dev)).cpu().numpy()
+        ref = _ref(oracle, qw, sc, su, sv, x, bias)
+        assert y.shape == ref.shape
+        err = _rel(y, ref)
+        worst = max(worst, err)
+        assert err <= REL_TOL, (case, m, n, K, M, dtype, with_bias, err)
+    print(f"sweep worst relative error {worst:.2e}", flush=True)

@@ -73,13 +73,15 @@ def test_dequant_q_bit_exact(dev, oracle, K):
     assert got.dtype == np.float32 and np.array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
+@pytest.mark.parametrize("shape", [(384, 256), (128, 128), (128, 640), (768, 128)])
 @pytest.mark.parametrize("K", [2, 3, 4, 5, 7])
-def test_dequant_w_original_basis(dev, oracle, K):
+def test_dequant_w_original_basis(dev, oracle, K, shape):
     from htr_amd import ops, wire
-    print(f"dequant_w K={K}", flush=True)
-    qw, sc, su, sv = wire.synth_linear(384, 256, K, 300 + K)
+    m, n = shape
+    print(f"dequant_w K={K} {m}x{n}", flush=True)
+    qw, sc, su, sv = wire.synth_linear(m, n, K, 300 + K + m)
     got = ops.dequant_w(*[t.to(dev) for t in (qw, sc, su, sv)])
-    assert got.dtype == torch.bfloat16 and tuple(got.shape) == (384, 256)
+    assert got.dtype == torch.bfloat16 and tuple(got.shape) == (m, n)
     ref = torch.from_numpy(oracle.c_dequant_w(qw.numpy(), sc.numpy(), su.numpy(), sv.numpy()))      # float64
     g = got.float().cpu().double()
     # bf16 rounding (2^-9 relative) of a value computed with float32 butterflies (error ~1e-6 of the block's scale)

@@ -338,20 +338,28 @@ __global__ __launch_bounds__(WG_THREADS) void k_rotate(const void* __restrict__ 
   const size_t row = (size_t)mrow * n;
   const int blk = blockIdx.x * WG_WAVES + w;
   const int col = blk * 128;
-  float va = 0.f, vb = 0.f;
-  if (blk < nblk) {                       // own block first: its loads overlap the scan
-    va = load_elem(x, x_dtype, row + col + lane) * sign_of(su, col + lane);
-    vb = load_elem(x, x_dtype, row + col + lane + 64) * sign_of(su, col + lane + 64);
-  }
-  // max|x| of the row.  |values| compare like their bit patterns, so the scan is integer: 16 bytes per thread and load
-  // through a descriptor over the row (pieces beyond its end read zeros), four loads in flight per thread.  Rows that
-  // are not 16-byte aligned take the element-wise loop.
-  float mx = 0.f;
-  const int es = x_dtype == HTR_F32 ? 4 : 2;
+  // Every load of the kernel goes out back to back, through descriptors over the activation row and the sign bytes:
+  // the wave's own block first (per element one 16-bit and one 32-bit load, the one that does not apply out of range:
+  // zeros, no traffic, no branch), then the scan of the whole row for max|x|.  Conversions come after the last load
+  // has been issued; a conversion between two loads makes the compiler wait for the first to return.
+  const bool is32 = x_dtype == HTR_F32, own = blk < nblk;
+  const int es = is32 ? 4 : 2;
   const unsigned char* xrow = (const unsigned char*)x + row * es;
+  const __amdgpu_buffer_rsrc_t rrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)xrow, 0, n * es, 0x00020000);
+  const __amdgpu_buffer_rsrc_t srsrc = __builtin_amdgcn_make_buffer_rsrc((void*)su, 0, n >> 3, 0x00020000);
+  constexpr int OUT_OF_RANGE = 0x7FFFFF00;
+  const int ea = col + lane, eb = ea + 64;
+  const uint32_t a16 = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rrsrc, own && !is32 ? ea * 2 : OUT_OF_RANGE, 0, 0);
+  const uint32_t b16 = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rrsrc, own && !is32 ? eb * 2 : OUT_OF_RANGE, 0, 0);
+  const uint32_t a32 = __builtin_amdgcn_raw_buffer_load_b32(rrsrc, own && is32 ? ea * 4 : OUT_OF_RANGE, 0, 0);
+  const uint32_t b32 = __builtin_amdgcn_raw_buffer_load_b32(rrsrc, own && is32 ? eb * 4 : OUT_OF_RANGE, 0, 0);
+  const uint32_t sa = (uint8_t)__builtin_amdgcn_raw_buffer_load_b8(srsrc, own ? ea >> 3 : OUT_OF_RANGE, 0, 0);
+  const uint32_t sb = (uint8_t)__builtin_amdgcn_raw_buffer_load_b8(srsrc, own ? eb >> 3 : OUT_OF_RANGE, 0, 0);
+  // max|x| of the row.  |values| compare like their bit patterns, so the scan is integer: 16 bytes per thread and load
+  // (pieces beyond the row's end read zeros), four loads in flight per thread.  Rows that are not 16-byte aligned are
+  // scanned element by element.
+  uint32_t m32 = 0u;            // float32: max of the sign-cleared words; 16-bit types: max of the sign-cleared halves
   if ((((size_t)xrow) & 15) == 0) {
-    const __amdgpu_buffer_rsrc_t rrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)xrow, 0, n * es, 0x00020000);
-    uint32_t m32 = 0u;          // float32: max of the sign-cleared words; 16-bit types: max of the sign-cleared halves
     for (int base = threadIdx.x * 16; base < n * es; base += 4 * WG_THREADS * 16) {
       u4 v[4];
 #pragma unroll
@@ -361,16 +369,26 @@ __global__ __launch_bounds__(WG_THREADS) void k_rotate(const void* __restrict__ 
         const uint32_t d[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
-          if (x_dtype == HTR_F32) m32 = max(m32, d[k] & 0x7FFFFFFFu);
+          if (is32) m32 = max(m32, d[k] & 0x7FFFFFFFu);
           else m32 = max(m32, max(d[k] & 0x7FFFu, (d[k] >> 16) & 0x7FFFu));
         }
       }
     }
-    mx = x_dtype == HTR_F32 ? __uint_as_float(m32) : x_dtype == HTR_BF16 ? bf16_bits_to_float((uint16_t)m32) : f16_bits_to_float((uint16_t)m32);
-    if (mx != mx) mx = __uint_as_float(0x7F800000u);   // a NaN anywhere: treat the row as unbounded (scale 1)
+  } else if (is32) {
+    for (int i = threadIdx.x; i < n; i += WG_THREADS)
+      m32 = max(m32, (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(rrsrc, i * 4, 0, 0) & 0x7FFFFFFFu);
   } else {
-    for (int i = threadIdx.x; i < n; i += WG_THREADS) mx = fmaxf(mx, fabsf(load_elem(x, x_dtype, row + i)));
+    for (int i = threadIdx.x; i < n; i += WG_THREADS)
+      m32 = max(m32, (uint32_t)(uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rrsrc, i * 2, 0, 0) & 0x7FFFu);
   }
+  float mx = is32 ? __uint_as_float(m32) : x_dtype == HTR_BF16 ? bf16_bits_to_float((uint16_t)m32) : f16_bits_to_float((uint16_t)m32);
+  if (mx != mx) mx = __uint_as_float(0x7F800000u);     // a NaN anywhere: treat the row as unbounded (scale 1)
+  // own elements: bits to float, input sign (bit j % 8 of byte j / 8 set: minus)
+  uint32_t abits = is32 ? a32 : x_dtype == HTR_BF16 ? a16 << 16 : __float_as_uint(f16_bits_to_float((uint16_t)a16));
+  uint32_t bbits = is32 ? b32 : x_dtype == HTR_BF16 ? b16 << 16 : __float_as_uint(f16_bits_to_float((uint16_t)b16));
+  abits ^= ((sa >> (ea & 7)) & 1u) << 31;
+  bbits ^= ((sb >> (eb & 7)) & 1u) << 31;
+  float va = __uint_as_float(abits), vb = __uint_as_float(bbits);
   mx = wave_max(mx);
   if (lane == 0) s_max[w] = mx;
   __syncthreads();

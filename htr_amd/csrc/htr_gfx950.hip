@@ -1530,7 +1530,7 @@ inline bool plan_for_chunk(int m, int n, int M, int chunk, Plan& pl) {
 
 // Picks the chunk length (virtual steps per workgroup) with a cost model in microseconds fitted to chunk-length sweeps
 // on MI355X (K4): a fixed latency chain (launch, x fetch, rotation, partial exchange, output rotation) that grows with
-// the contributors a finisher reads; a cost per step that depends on how many workgroups share a CU (one: latency
+// the contributors a finisher reads, eight per round trip; a cost per step that depends on how many workgroups share a CU (one: latency
 // bound, cheaper on a part-filled chip, dearer for long chunks; several: throughput bound, proportional to the
 // load of the fullest CU); a penalty for chunks that do not tile the rows of column blocks; the extra launch of a
 // pre-rotation; and the growth of all per-step work with the number of activation rows.
@@ -1563,7 +1563,9 @@ inline bool make_plan(int m, int n, int M, int nsplit, Plan& pl) {
     const double fill2 = fill < 1.5 ? 1.5 : fill;
     const double body = fill <= 1.0 ? rows * (0.25 + 0.3 * fill + 0.008 * chunk) * steps
                                     : fill2 * (rows * 0.6 * steps + 0.5 + 0.3 * M);
-    const double t = 4.5 + 0.06 * contributors + (c.prerot ? 3.0 : 0.0) + body;
+    // hand-over: every contributor's slot is read (0.03 us each), eight per round trip to memory (0.45 us each)
+    const double handover = 0.03 * contributors + 0.45 * ((contributors - 1 + 7) / 8);
+    const double t = 4.5 + handover + (c.prerot ? 3.0 : 0.0) + body;
     if (t < best) { best = t; pl = c; found = true; }
   }
   return found;

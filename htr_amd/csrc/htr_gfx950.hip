@@ -29,6 +29,7 @@
 #include <stdint.h>
 #include <string.h>
 #include <stdlib.h>
+#include <type_traits>
 
 #include "../../include/htr_gfx950.h"
 
@@ -278,7 +279,7 @@ struct LinearTail {
   const void* bias;
   void* y;
   const _Float16* xt_g;   // pre-rotated activations [M][n] f16 (only when PREROT)
-  const float* xs_g;      // their per-(row, block, tile parity) sums [M][n/128][2]
+  const float* xs_g;      // their sums per (row, block) [M][n/128][4]: even tiles, odd tiles, columns 0..63, columns 64..127
   const float* sc_g;      // per-row activation scale [M]
   uint32_t* status;       // workspace word that collects kernel-side failures (bit 0: a finisher gave up waiting)
   unsigned long long chunk_magic;   // ceil(2^40 / chunk): step index -> chunk index
@@ -404,9 +405,12 @@ __global__ __launch_bounds__(WG_THREADS) void k_rotate(const void* __restrict__ 
     const _Float16 ha = (_Float16)(va * INV_SQRT128), hb = (_Float16)(vb * INV_SQRT128);
     xt_g[row + col + lane] = ha;
     xt_g[row + col + lane + 64] = hb;
-    float se, so;
-    wave_sum_by_row_parity((float)ha + (float)hb, se, so);
-    if (lane == 0) { xs_g[((size_t)mrow * nblk + blk) * 2] = se; xs_g[((size_t)mrow * nblk + blk) * 2 + 1] = so; }
+    // sums of the rounded values: the lane's first element lies in tile lane / 16, its second in tile 4 + lane / 16, so the
+    // 16-lane row parity is the tile parity of both, and the two elements are the two halves of the block
+    float ea, oa, eb, ob;
+    wave_sum_by_row_parity((float)ha, ea, oa);
+    wave_sum_by_row_parity((float)hb, eb, ob);
+    if (lane == 0) *(f4*)(xs_g + ((size_t)mrow * nblk + blk) * 4) = f4{ea + eb, oa + ob, ea + oa, eb + ob};
   }
 }
 
@@ -697,7 +701,7 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
     }
     for (int i = threadIdx.x; i < npairs * 2; i += WG_THREADS) {
       const int pi = i >> 1, mrow = row_of_pair(pi), li = pi - mrow * nbl;
-      s_xs[i] = t.xs_g[((size_t)mrow * nblk + (pair_col(li) >> 7)) * 2 + (i & 1)];
+      s_xs[i] = t.xs_g[((size_t)mrow * nblk + (pair_col(li) >> 7)) * 4 + (i & 1)];
     }
   }
 #pragma unroll
@@ -915,14 +919,32 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
 // LDS next to useful chunk lengths, and short chunks mean that every workgroup copies a large activation slice and
 // hands over a large partial for little weight traffic.  Here a workgroup owns one 128-row block and 1/S of its
 // column blocks (grid = S x row blocks), and the activations (rotated ahead by k_rotate) are staged through LDS one
-// 128-column block at a time, double-buffered, one barrier per step; the decoded weights of a step feed MB * 4 matrix
-// instructions.  The split S along the columns is only as large as filling the chip needs; S = 1 needs no exchange.
-template <int K, int MB, int P>
+// 128-column block at a time, double-buffered, one barrier per step.  The split S along the columns is only as large
+// as filling the chip needs; S = 1 needs no exchange.
+//   wave    = two adjacent 16-row strips (pair sp = w / 2) x one half (ch = w % 2) of the block's columns: 2 x 4 tiles
+//             per step, two runs of 128 K contiguous bytes
+//   lane    = (tile column g = lane / 16, strip h = lane / 8 % 2, row pair q = lane % 8); a tile is still 8 consecutive
+//             lanes, so the decode is the one of k_linear
+//   product = MFMA row i = lane % 16 = (h, q): rows 2q (or 2q + 1) of both strips, all of them over the same 32 columns
+//             (k-slot g = columns 0..7, or 8..15, of tile column 4 ch + g).  So every one of the 16 MFMA columns carries
+//             an activation row: 16 rows per matrix instruction, and a wave reads only its half of the block from LDS.
+//             D[i][c] sits in lane c + 16 * (i / 4), register i % 4: lane (g', c) ends up with rows 32 sp + 8 g' .. + 7
+//             of the row block for activation row c.
+//   The two waves of a strip pair leave their column halves side by side in LDS when the split is done; whoever reads
+//   the workgroup's partial adds the two.
+constexpr int BATCH_ROWH = 128 + 8;          // halves per staged activation row: 16 rows x 16 bytes then cover every bank once
+constexpr int BATCH_FIN_STRIDE = 128 + 4;    // floats per activation row of the workgroup's partial
+// position of output row r (0..127) in a row of the partial: [r % 8][r / 8], so that the lanes of a wave (16 activation
+// rows x 4 groups of 8 output rows) hit 64 different banks with each of their 8 values
+__device__ __forceinline__ int batch_fin_pos(int r) { return (r & 7) * 16 + (r >> 3); }
+
+template <int K, int MG, int P>
 __global__ __launch_bounds__(WG_THREADS) void k_linear_batch(const uint32_t* __restrict__ qw, float* __restrict__ part,
                                                              int m, int n, int M, int S, int flags, const LinearTail t) {
   extern __shared__ __align__(16) unsigned char lds[];
   const int lane = threadIdx.x & 63;
   const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int sp = w >> 1, ch = w & 1;
   const int nblk = n >> 7;
   const int s_idx = blockIdx.x, rb = blockIdx.y;
   const int cb = (nblk + S - 1) / S;                               // column blocks per split
@@ -930,8 +952,8 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear_batch(const uint32_t* __r
   const int nsteps = c_end - c_begin;                              // >= 1: the host picks S so that no split is empty
   const int y_dtype = (flags >> 2) & 3;
 
-  // LDS: [2 buffers][(M + 1) rows][144 halves] x~ blocks, [2][2 M] sums, [M][128] partials of the finishing workgroup
-  constexpr int ROWH = 128 + 16;
+  // LDS: [2 buffers][(M + 1) rows][136 halves] x~ blocks, [2][2 M] sums, [2 column halves][M][132] partial of the workgroup
+  constexpr int ROWH = BATCH_ROWH;
   const int bufh = (M + 1) * ROWH;
   _Float16* xt = (_Float16*)lds;
   float* s_xs = (float*)(lds + (size_t)2 * bufh * 2);
@@ -942,7 +964,7 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear_batch(const uint32_t* __r
   const bool has_piece = tid < M * 16, has_sum = tid < 2 * M;
   const int p_row = tid >> 4, p_idx = tid & 15;
   const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)t.xt_g, 0, M * n * 2, 0x00020000);
-  const __amdgpu_buffer_rsrc_t srsrc = __builtin_amdgcn_make_buffer_rsrc((void*)t.xs_g, 0, M * nblk * 8, 0x00020000);
+  const __amdgpu_buffer_rsrc_t srsrc = __builtin_amdgcn_make_buffer_rsrc((void*)t.xs_g, 0, M * nblk * 16, 0x00020000);
   constexpr int OUT_OF_RANGE = 0x7FFFFF00;
   const int piece_lds = p_row * ROWH + (p_idx & 1) * 64 + (p_idx >> 1) * 8;        // halves, inside a buffer
   // Blocks travel two steps ahead of their use in two register sets (q = block parity): loads return in order, so
@@ -954,7 +976,8 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear_batch(const uint32_t* __r
     HTR_PIN();
     const bool live = blk < c_end;
     xg[q] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, live && has_piece ? (p_row * n + blk * 128 + p_idx * 8) * 2 : OUT_OF_RANGE, 0, 0);
-    xsg[q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(srsrc, live && has_sum ? (((tid >> 1) * nblk + blk) * 2 + (tid & 1)) * 4 : OUT_OF_RANGE, 0, 0));
+    // sums over columns 0..63 and 64..127 of the block: entries 2 and 3 of the block's four
+    xsg[q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(srsrc, live && has_sum ? (((tid >> 1) * nblk + blk) * 4 + 2 + (tid & 1)) * 4 : OUT_OF_RANGE, 0, 0));
     HTR_PIN();
   };
   auto stage_store = [&](int q) {            // block of parity q goes to buffer q
@@ -984,50 +1007,55 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear_batch(const uint32_t* __r
     }
   }
 
-  // ---- the weight stream of this wave: one contiguous piece of its strip
+  // ---- the weight stream of this wave: per step, tiles 4 ch .. 4 ch + 3 of strips 2 sp and 2 sp + 1.  One descriptor
+  // from the first strip's first byte of the split to the second strip's last: lanes of the second strip that run past
+  // the split are out of range (zeros, no traffic); lanes of the first strip would land in later column blocks, so a
+  // request beyond the last step is sent out of range as a whole.
   constexpr int STEP_BYTES = 256 * K;
-  const uint32_t* wave_base = qw + ((size_t)(rb * 8 + w) * nblk + (size_t)c_begin) * (STEP_BYTES / 4);
-  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)wave_base, 0, nsteps * STEP_BYTES, 0x00020000);
-  int pf_off = lane * 4 * K;
+  const uint32_t strip_bytes = (uint32_t)nblk * STEP_BYTES;
+  const uint32_t* wave_base = qw + ((size_t)(rb * 8 + 2 * sp) * nblk + (size_t)c_begin) * (STEP_BYTES / 4);
+  const __amdgpu_buffer_rsrc_t rsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void*)wave_base, 0, (int)(strip_bytes + (uint32_t)nsteps * STEP_BYTES), 0x00020000);
+  const int g = lane >> 4, n16 = lane & 15;
+  int pf_off = ((lane >> 3) & 1) * (int)strip_bytes + ((4 * ch + g) * 8 + (lane & 7)) * 4 * K;
+  int pf_left = nsteps;                      // steps not yet requested (uniform)
   StreamRegs<K> buf[P];
   auto prefetch = [&](StreamRegs<K>& dst) {
     HTR_PIN();
-    load_stream_buffer<K>(rsrc, pf_off, dst);
+    load_stream_buffer<K>(rsrc, pf_left > 0 ? pf_off : OUT_OF_RANGE, dst);
     pf_off += STEP_BYTES;
+    --pf_left;
     HTR_PIN();
   };
 #pragma unroll
   for (int p = 0; p < P; ++p) prefetch(buf[p]);
 
-  // ---- per-lane constants of the product (as in k_linear)
-  const int g = lane >> 4, n16 = lane & 15;
-  const int par = g >> 1;
-  const bool mine = (n16 & 1) == par;
-  int boff[MB], xsoff[MB];
-  float sc[MB], offs[MB], k1534[MB];
+  // ---- per-lane constants of the product: this lane's B operands and sums belong to activation row 16 mg + lane % 16
+  int boff[MG], xsoff[MG];
+  float sc[MG], offs[MG], k1534[MG];
 #pragma unroll
-  for (int mb = 0; mb < MB; ++mb) {
-    const int mrow = mb * 8 + (n16 >> 1);
-    const bool live = mine && mrow < M;
-    boff[mb] = (mrow < M ? mrow : M) * ROWH + 8 * (2 * g + (n16 & 1));
-    xsoff[mb] = live ? 2 * mrow + par : -1;
-    offs[mb] = 0.f;
-    sc[mb] = live ? t.sc_g[mrow] : 0.f;
-    k1534[mb] = live ? 1534.f : 0.f;
+  for (int mg = 0; mg < MG; ++mg) {
+    const int mrow = mg * 16 + n16;
+    const bool live = mrow < M;
+    boff[mg] = (live ? mrow : M) * ROWH + 8 * (4 * ch + g);
+    xsoff[mg] = live ? 2 * mrow + ch : 0;
+    offs[mg] = 0.f;
+    sc[mg] = live ? t.sc_g[mrow] : 0.f;
+    k1534[mg] = live ? 1534.f : 0.f;
   }
-  f4 acc[MB][2];
+  f4 acc[MG][2];
 #pragma unroll
-  for (int mb = 0; mb < MB; ++mb) { acc[mb][0] = f4{0.f, 0.f, 0.f, 0.f}; acc[mb][1] = f4{0.f, 0.f, 0.f, 0.f}; }
+  for (int mg = 0; mg < MG; ++mg) { acc[mg][0] = f4{0.f, 0.f, 0.f, 0.f}; acc[mg][1] = f4{0.f, 0.f, 0.f, 0.f}; }
 
-  h8 B0[MB], B1[MB];
-  float xsv[MB];
+  h8 B0[MG], B1[MG];
+  float xsv[MG];
   auto load_b = [&](int bsel) {
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-      const _Float16* bp = xt + bsel * bufh + boff[mb];
-      B0[mb] = *(const h8*)bp;
-      B1[mb] = *(const h8*)(bp + 64);
-      xsv[mb] = s_xs[bsel * 2 * M + max(xsoff[mb], 0)];
+    for (int mg = 0; mg < MG; ++mg) {
+      const _Float16* bp = xt + bsel * bufh + boff[mg];
+      B0[mg] = *(const h8*)bp;
+      B1[mg] = *(const h8*)(bp + 64);
+      xsv[mg] = s_xs[bsel * 2 * M + xsoff[mg]];
     }
   };
 
@@ -1044,15 +1072,15 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear_batch(const uint32_t* __r
 
   auto multiply = [&](const DecodedStep<K>& d) {
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) acc[mb][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[0], B0[mb], acc[mb][0], 0, 0, 0);
+    for (int mg = 0; mg < MG; ++mg) acc[mg][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[0], B0[mg], acc[mg][0], 0, 0, 0);
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) acc[mb][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[2], B0[mb], acc[mb][1], 0, 0, 0);
+    for (int mg = 0; mg < MG; ++mg) acc[mg][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[2], B0[mg], acc[mg][1], 0, 0, 0);
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) acc[mb][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[1], B1[mb], acc[mb][0], 0, 0, 0);
+    for (int mg = 0; mg < MG; ++mg) acc[mg][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[1], B1[mg], acc[mg][0], 0, 0, 0);
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) acc[mb][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[3], B1[mb], acc[mb][1], 0, 0, 0);
+    for (int mg = 0; mg < MG; ++mg) acc[mg][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[3], B1[mg], acc[mg][1], 0, 0, 0);
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) offs[mb] = __builtin_fmaf(k1534[mb], xsv[mb], offs[mb]);
+    for (int mg = 0; mg < MG; ++mg) offs[mg] = __builtin_fmaf(k1534[mg], xsv[mg], offs[mg]);
   };
   // One step with a successor: multiply step v, put the block of step v + 1 (in registers since the previous step)
   // into the other buffer, request the block of step v + 2, decode step v + 1; between the two halves of the decode
@@ -1075,35 +1103,31 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear_batch(const uint32_t* __r
     else if (v + pp < nsteps) multiply(cur);
   }
 
-  // ---- this wave's strip partial per activation row: offset removed, activation scale undone, tile parities added
+  // ---- this wave's partial (offset removed, activation scale undone) goes to its column half's copy in LDS
 #pragma unroll
-  for (int mb = 0; mb < MB; ++mb) {
-    const int mrow = mb * 8 + (n16 >> 1);
-    float tot[8];
+  for (int mg = 0; mg < MG; ++mg) {
+    const int mrow = mg * 16 + n16;
+    if (mrow < M) {
+      float* dst = s_fin + (ch * M + mrow) * BATCH_FIN_STRIDE + 4 * sp + g;       // row 32 sp + 8 g + i sits at i * 16 + 4 sp + g
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+      for (int j = 0; j < 4; ++j)
 #pragma unroll
-      for (int rr = 0; rr < 2; ++rr) {
-        const float val = xsoff[mb] >= 0 ? (acc[mb][rr][j] - offs[mb]) * sc[mb] : 0.f;
-        float lo_half, hi_half;
-        halves32(lane_xor_dpp<1>(val), lo_half, hi_half);
-        tot[2 * j + rr] = val + hi_half;
-      }
-    if (lane < 32 && (n16 & 1) == 0 && mrow < M) {
-      const int rowi = 16 * w + 8 * (g & 1);
-      if (finisher) {
-        float* dst = s_fin + (size_t)mrow * 128 + rowi;
-        *(f4*)dst = f4{tot[0], tot[1], tot[2], tot[3]};
-        *(f4*)(dst + 4) = f4{tot[4], tot[5], tot[6], tot[7]};
-      } else {
-        uint32_t* dst = (uint32_t*)(part + (((size_t)rb * S + s_idx) * M + mrow) * 128 + rowi);
-#pragma unroll
-        for (int i = 0; i < 8; ++i)
-          __hip_atomic_store(dst + i, __float_as_uint(tot[i]) | 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      }
+        for (int rr = 0; rr < 2; ++rr)
+          dst[(2 * j + rr) * 16] = (acc[mg][rr][j] - offs[mg]) * sc[mg];
     }
   }
-  if (!finisher) return;
+  __syncthreads();
+  const int pos0 = batch_fin_pos(lane), pos1 = batch_fin_pos(lane + 64);
+  if (!finisher) {
+    for (int mrow = w; mrow < M; mrow += WG_WAVES) {
+      const float* own = s_fin + mrow * BATCH_FIN_STRIDE;
+      const float* oth = own + M * BATCH_FIN_STRIDE;
+      uint32_t* dst = (uint32_t*)(part + (((size_t)rb * S + s_idx) * M + mrow) * 128);
+      __hip_atomic_store(dst + lane, __float_as_uint(own[pos0] + oth[pos0]) | 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(dst + lane + 64, __float_as_uint(own[pos1] + oth[pos1]) | 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    return;
+  }
 
   // ---- output side: the last split of the row block adds the other splits' partials (fixed order) and finishes
   const float rs0 = f16_bits_to_float((uint16_t)raw_sc0) * t.cbscale * INV_SQRT128;
@@ -1113,38 +1137,39 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear_batch(const uint32_t* __r
     return y_dtype == HTR_F32 ? __uint_as_float(b) : y_dtype == HTR_BF16 ? bf16_bits_to_float((uint16_t)b) : f16_bits_to_float((uint16_t)b);
   };
   const float b0v = cvt_bias(raw_b0), b1v = cvt_bias(raw_b1);
-  __syncthreads();
-  for (int mrow = w; mrow < M; mrow += WG_WAVES) {
-    float v0s = 0.f, v1s = 0.f;
-    bool failed = false;
-    if (S > 1) {
-      int tries = 0;
-      for (;;) {
-        bool missing = false;
-        v0s = 0.f; v1s = 0.f;
-        for (int jb = 0; jb < S - 1; jb += 8) {
-          uint32_t u0[8], u1[8];
+  auto slot_of = [&](int j, int mrow) { return (uint32_t*)(part + (((size_t)rb * S + j) * M + mrow) * 128); };
+  // waits (bounded) until every other split's partial of activation row mrow is there; their sum in fixed order
+  auto wait_for_row = [&](int mrow, float& v0s, float& v1s) {
+    int tries = 0;
+    for (;;) {
+      bool missing = false;
+      v0s = 0.f; v1s = 0.f;
+      for (int jb = 0; jb < S - 1; jb += 8) {
+        uint32_t u0[8], u1[8];
 #pragma unroll
-          for (int k = 0; k < 8; ++k) {
-            const int j = min(jb + k, S - 2);
-            const uint32_t* pp = (const uint32_t*)(part + (((size_t)rb * S + j) * M + mrow) * 128);
-            u0[k] = __hip_atomic_load(pp + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            u1[k] = __hip_atomic_load(pp + lane + 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          }
-#pragma unroll
-          for (int k = 0; k < 8; ++k)
-            if (jb + k < S - 1) {
-              missing |= (u0[k] == 0u) | (u1[k] == 0u);
-              v0s += __uint_as_float(u0[k]); v1s += __uint_as_float(u1[k]);
-            }
+        for (int k = 0; k < 8; ++k) {
+          const uint32_t* pp = slot_of(min(jb + k, S - 2), mrow);
+          u0[k] = __hip_atomic_load(pp + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          u1[k] = __hip_atomic_load(pp + lane + 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        if (!__any(missing)) break;
-        if (++tries >= t.spin_limit) { failed = true; break; }
-        __builtin_amdgcn_s_sleep(2);
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+          if (jb + k < S - 1) {
+            missing |= (u0[k] == 0u) | (u1[k] == 0u);
+            v0s += __uint_as_float(u0[k]); v1s += __uint_as_float(u1[k]);
+          }
       }
+      if (!__any(missing)) return false;
+      if (++tries >= t.spin_limit) return true;
+      __builtin_amdgcn_s_sleep(2);
+    }
+  };
+  // the rest of a row: slots back to zero for the next call (or the failure noted), own partial, output side
+  auto finish_row = [&](int mrow, float v0s, float v1s, bool failed) {
+    if (S > 1) {
       if (!failed) {
         for (int j = 0; j < S - 1; ++j) {
-          uint32_t* pp = (uint32_t*)(part + (((size_t)rb * S + j) * M + mrow) * 128);
+          uint32_t* pp = slot_of(j, mrow);
           __hip_atomic_store(pp + lane, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           __hip_atomic_store(pp + lane + 64, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
@@ -1152,8 +1177,9 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear_batch(const uint32_t* __r
         __hip_atomic_fetch_or(t.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
     }
-    const float* own = s_fin + (size_t)mrow * 128;
-    v0s += own[lane]; v1s += own[lane + 64];
+    const float* own = s_fin + mrow * BATCH_FIN_STRIDE;
+    const float* oth = own + M * BATCH_FIN_STRIDE;
+    v0s += own[pos0] + oth[pos0]; v1s += own[pos1] + oth[pos1];
     v0s *= rs0; v1s *= rs1;
     fwht128_wave(v0s, v1s, lane);
     v0s = __builtin_fmaf(v0s, sg0, b0v);
@@ -1161,6 +1187,63 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear_batch(const uint32_t* __r
     if (failed) { v0s = __builtin_nanf(""); v1s = v0s; }
     store_elem_g(t.y, y_dtype, (size_t)mrow * m + r0, v0s);
     store_elem_g(t.y, y_dtype, (size_t)mrow * m + r1, v1s);
+  };
+  // Wave w finishes activation rows w, w + 8, ...
+  constexpr int RPW = MG * 16 / WG_WAVES;        // rows per wave at most
+  if (w >= M) return;
+  // With up to eight other splits, all of the wave's rows are polled together, so that the rows behind the first cost
+  // no memory round trip of their own.  JW = slots requested per row (the next power of two from S - 1; the surplus
+  // repeats the last slot).
+  auto finish_rows_together = [&](auto jw) {
+    constexpr int JW = decltype(jw)::value;
+    float a0[RPW], a1[RPW];
+    int tries = 0;
+    bool failed = false;
+    for (;;) {
+      uint32_t u0[RPW][JW], u1[RPW][JW];
+#pragma unroll
+      for (int r = 0; r < RPW; ++r)
+#pragma unroll
+        for (int k = 0; k < JW; ++k) {
+          const uint32_t* pp = slot_of(min(k, S - 2), min(w + r * WG_WAVES, M - 1));
+          u0[r][k] = __hip_atomic_load(pp + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          u1[r][k] = __hip_atomic_load(pp + lane + 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      bool missing = false;
+#pragma unroll
+      for (int r = 0; r < RPW; ++r) {
+        a0[r] = 0.f; a1[r] = 0.f;
+#pragma unroll
+        for (int k = 0; k < JW; ++k)
+          if (k < S - 1) {
+            missing |= (u0[r][k] == 0u) | (u1[r][k] == 0u);
+            a0[r] += __uint_as_float(u0[r][k]); a1[r] += __uint_as_float(u1[r][k]);
+          }
+      }
+      if (!__any(missing)) break;
+      if (++tries >= t.spin_limit) { failed = true; break; }
+      __builtin_amdgcn_s_sleep(2);
+    }
+#pragma unroll
+    for (int r = 0; r < RPW; ++r)
+      if (w + r * WG_WAVES < M) finish_row(w + r * WG_WAVES, a0[r], a1[r], failed);
+  };
+  if (S > 1 && S - 1 <= 8 && w + WG_WAVES < M) {
+    if (S - 1 <= 1) finish_rows_together(std::integral_constant<int, 1>{});
+    else if (S - 1 <= 2) finish_rows_together(std::integral_constant<int, 2>{});
+    else if (S - 1 <= 4) finish_rows_together(std::integral_constant<int, 4>{});
+    else finish_rows_together(std::integral_constant<int, 8>{});
+    return;
+  }
+  {
+    float v0s = 0.f, v1s = 0.f;
+    const bool failed = S > 1 ? wait_for_row(w, v0s, v1s) : false;
+    finish_row(w, v0s, v1s, failed);
+  }
+  for (int mrow = w + WG_WAVES; mrow < M; mrow += WG_WAVES) {
+    float v0s = 0.f, v1s = 0.f;
+    const bool failed = S > 1 ? wait_for_row(mrow, v0s, v1s) : false;
+    finish_row(mrow, v0s, v1s, failed);
   }
 }
 
@@ -1501,7 +1584,7 @@ inline size_t ws_need(size_t slot_bytes, size_t scratch_bytes) {
 }
 inline size_t ws_half(size_t workspace_bytes) { return workspace_bytes / 2 / 256 * 256; }
 // bytes of the pre-rotated activations, their block sums and the row scales
-inline size_t prerot_bytes(int n, int M) { return align256((size_t)M * n * 2) + align256((size_t)M * (n / 128) * 8) + align256((size_t)M * 4); }
+inline size_t prerot_bytes(int n, int M) { return align256((size_t)M * n * 2) + align256((size_t)M * (n / 128) * 16) + align256((size_t)M * 4); }
 
 constexpr int NUM_CU = 256;
 constexpr int MAX_ROW_BLOCKS = 16384;
@@ -1619,11 +1702,11 @@ template <int K> int launch_linear_k(const LinearLaunch& a, bool prerot, int mb,
 
 // ---- batched kernel: split S of the column blocks per row block
 struct BatchPlan { int S, cb, wgs, mb; size_t lds; };
-constexpr int BATCH_MIN_M = 8;      // rows from which the library policy takes the batched kernel
-inline size_t batch_lds_bytes(int M) { return (size_t)2 * (M + 1) * (128 + 16) * 2 + (size_t)4 * M * 4 + (size_t)M * 128 * 4; }
+constexpr int BATCH_MIN_M = 6;      // rows from which the library policy takes the batched kernel
+inline size_t batch_lds_bytes(int M) { return (size_t)2 * (M + 1) * BATCH_ROWH * 2 + (size_t)4 * M * 4 + (size_t)2 * M * BATCH_FIN_STRIDE * 4; }
 inline bool make_batch_plan(int m, int n, int M, int want_S, BatchPlan& bp) {
   const int nblk = n / 128, rbs = m / 128;
-  bp.mb = M <= 8 ? 1 : (M <= 16 ? 2 : 4);
+  bp.mb = M <= 16 ? 1 : 2;                  // groups of 16 activation rows
   bp.lds = batch_lds_bytes(M);
   // Measured on MI355X (K4, 8..32 rows, 4096..28672 output rows): one workgroup per CU is the best fill; every further
   // split adds partial traffic that grows with the rows.  So: the largest split that keeps the grid within the CU
@@ -1661,8 +1744,7 @@ template <int K> int launch_batch_k(const uint32_t* qw, float* part, int m, int 
                                     const BatchPlan& bp, hipStream_t st) {
   switch (bp.mb) {
     case 1: return launch_batch_v<K, 1>(qw, part, m, n, M, flags, t, bp, st);
-    case 2: return launch_batch_v<K, 2>(qw, part, m, n, M, flags, t, bp, st);
-    default: return launch_batch_v<K, 4>(qw, part, m, n, M, flags, t, bp, st);
+    default: return launch_batch_v<K, 2>(qw, part, m, n, M, flags, t, bp, st);
   }
 }
 // nsplit bit 29: batched kernel with the split in the low bits (0 = policy); otherwise the policy decides by M
@@ -1760,7 +1842,7 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
     t.scales = (const uint16_t*)scales; t.sv = (const uint8_t*)sv; t.bias = bias; t.y = y;
     t.xt_g = (const _Float16*)wsp;
     t.xs_g = (const float*)(wsp + align256((size_t)M * n * 2));
-    t.sc_g = (const float*)(wsp + align256((size_t)M * n * 2) + align256((size_t)M * (n / 128) * 8));
+    t.sc_g = (const float*)(wsp + align256((size_t)M * n * 2) + align256((size_t)M * (n / 128) * 16));
     t.status = (uint32_t*)workspace;
     t.cbscale = htr_cbscale();
     t.spin_limit = g_spin_limit;
@@ -1811,7 +1893,7 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
   if (prerot) {
     t.xt_g = (const _Float16*)wsp;
     t.xs_g = (const float*)(wsp + align256((size_t)M * n * 2));
-    t.sc_g = (const float*)(wsp + align256((size_t)M * n * 2) + align256((size_t)M * (n / 128) * 8));
+    t.sc_g = (const float*)(wsp + align256((size_t)M * n * 2) + align256((size_t)M * (n / 128) * 16));
     hipLaunchKernelGGL(k_rotate, dim3((n / 128 + WG_WAVES - 1) / WG_WAVES, M), dim3(WG_THREADS), 0, st, x, (const uint8_t*)su, n, x_dtype, (_Float16*)t.xt_g,
                        (float*)t.xs_g, (float*)t.sc_g, (const htr_group_entry*)nullptr, 0ull);
     hipError_t e = hipGetLastError();
@@ -1877,7 +1959,7 @@ int htr_linear_grouped(const htr_group_entry* entries, int count, int m, int n, 
   t.scales = nullptr; t.sv = nullptr; t.bias = nullptr; t.y = nullptr;
   t.xt_g = (const _Float16*)wsp;
   t.xs_g = (const float*)(wsp + align256((size_t)max_M * n * 2));
-  t.sc_g = (const float*)(wsp + align256((size_t)max_M * n * 2) + align256((size_t)max_M * (n / 128) * 8));
+  t.sc_g = (const float*)(wsp + align256((size_t)max_M * n * 2) + align256((size_t)max_M * (n / 128) * 16));
   t.status = (uint32_t*)workspace;
   t.cbscale = htr_cbscale();
   t.spin_limit = g_spin_limit;

@@ -176,7 +176,7 @@ def prefill(dev):
         W = ops.dequant_w(*w)
         row = {"m": m, "n": n, "K": 4, "dequant_w_us": round(td, 1),
                "dequant_w_written_GBps": round(2.0 * m * n / td / 1e3, 1), "rows": []}
-        for M in (32, 64, 128, 512):
+        for M in (32, 64, 128, 256, 512):
             x = wire.synth_activation(M, n, SEED + 3, torch.bfloat16, dev)
             tg = eager(lambda: torch.nn.functional.linear(x, W))
             old, ops.GEMV_LOOP_MAX = ops.GEMV_LOOP_MAX, 10 ** 9

@@ -952,44 +952,59 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear_batch(const uint32_t* __r
   const int nsteps = c_end - c_begin;                              // >= 1: the host picks S so that no split is empty
   const int y_dtype = (flags >> 2) & 3;
 
-  // LDS: [2 buffers][(M + 1) rows][136 halves] x~ blocks, [2][2 M] sums, [2 column halves][M][132] partial of the workgroup
-  constexpr int ROWH = BATCH_ROWH;
-  const int bufh = (M + 1) * ROWH;
+  // LDS: [2 buffers][16 MG rows][136 halves] x~ blocks, [2][16 MG][2] sums, [16 MG] activation scales,
+  // [2 column halves][M][132] partial of the workgroup.  Rows M .. 16 MG - 1 are staged like the others (they read out of
+  // range: zeros), so every group of 16 rows is addressed alike.  With more than 64 rows the partial does not fit
+  // behind the blocks and takes their place once the last step is done.
+  constexpr int ROWH = BATCH_ROWH, ROWS = 16 * MG, BUFH = ROWS * ROWH;
+  constexpr bool FIN_OVER_BLOCKS = MG > 4;
   _Float16* xt = (_Float16*)lds;
-  float* s_xs = (float*)(lds + (size_t)2 * bufh * 2);
-  float* s_fin = s_xs + 4 * M;
+  float* s_xs = (float*)(lds + (size_t)2 * BUFH * 2);
+  float* s_sc = s_xs + 4 * ROWS;
+  float* s_fin = FIN_OVER_BLOCKS ? (float*)lds : s_sc + ROWS;
 
-  // ---- activation staging: thread = one 16-byte piece (8 halves) of the block: row tid / 16, piece tid % 16
+  // ---- activation staging in 16-byte pieces (8 halves): piece pi of the block is row pi / 16, columns 8 (pi % 16) .. + 7;
+  // a thread takes pieces tid, tid + 512, ...
+  constexpr int NPT = MG >= 2 ? MG / 2 : 1;      // pieces per thread
   const int tid = threadIdx.x;
-  const bool has_piece = tid < M * 16, has_sum = tid < 2 * M;
-  const int p_row = tid >> 4, p_idx = tid & 15;
+  const bool has_piece = MG >= 2 || tid < ROWS * 16, has_sum = tid < 2 * ROWS;
   const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)t.xt_g, 0, M * n * 2, 0x00020000);
   const __amdgpu_buffer_rsrc_t srsrc = __builtin_amdgcn_make_buffer_rsrc((void*)t.xs_g, 0, M * nblk * 16, 0x00020000);
   constexpr int OUT_OF_RANGE = 0x7FFFFF00;
-  const int piece_lds = p_row * ROWH + (p_idx & 1) * 64 + (p_idx >> 1) * 8;        // halves, inside a buffer
-  // Blocks travel two steps ahead of their use in two register sets (q = block parity): loads return in order, so
-  // waiting for a block also waits for every weight load issued before it, and one step of distance would cut the
-  // weight stream's run-ahead to a single step.
-  u4 xg[2];
-  float xsg[2];
+  int piece_lds[NPT], piece_src[NPT];            // halves inside a buffer; byte offset in x~ of the piece in block 0
+#pragma unroll
+  for (int i = 0; i < NPT; ++i) {
+    const int pi = tid + i * WG_THREADS, p_row = pi >> 4, p_idx = pi & 15;
+    piece_lds[i] = p_row * ROWH + (p_idx & 1) * 64 + (p_idx >> 1) * 8;
+    piece_src[i] = p_row < M ? (p_row * n + p_idx * 8) * 2 : -1;
+  }
+  const int sum_src = (tid >> 1) < M ? (((tid >> 1) * nblk) * 4 + 2 + (tid & 1)) * 4 : -1;   // sums over columns 0..63 | 64..127
+  // Blocks travel ahead of their use in registers: two steps (two register sets, by block parity) up to 32 rows, because
+  // loads return in order, so that waiting for a block also waits for every weight load issued before it, and one step
+  // of distance would cut the weight stream's run-ahead to a single step; with more rows a step is long enough for one.
+  constexpr int DIST = MG <= 2 ? 2 : 1;
+  u4 xg[DIST][NPT];
+  float xsg[DIST];
   auto stage_load = [&](int blk, int q) {    // block index in the row; beyond the split: zeros, no traffic
     HTR_PIN();
     const bool live = blk < c_end;
-    xg[q] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, live && has_piece ? (p_row * n + blk * 128 + p_idx * 8) * 2 : OUT_OF_RANGE, 0, 0);
-    // sums over columns 0..63 and 64..127 of the block: entries 2 and 3 of the block's four
-    xsg[q] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(srsrc, live && has_sum ? (((tid >> 1) * nblk + blk) * 4 + 2 + (tid & 1)) * 4 : OUT_OF_RANGE, 0, 0));
+    const int set = DIST == 2 ? q : 0;
+#pragma unroll
+    for (int i = 0; i < NPT; ++i)
+      xg[set][i] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, live && piece_src[i] >= 0 ? piece_src[i] + blk * 256 : OUT_OF_RANGE, 0, 0);
+    xsg[set] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(srsrc, live && sum_src >= 0 ? sum_src + blk * 16 : OUT_OF_RANGE, 0, 0));
     HTR_PIN();
   };
-  auto stage_store = [&](int q) {            // block of parity q goes to buffer q
-    if (has_piece) *(u4*)(xt + q * bufh + piece_lds) = xg[q];
-    if (has_sum) s_xs[q * 2 * M + tid] = xsg[q];
+  auto stage_store = [&](int q) {            // the block of parity q goes to buffer q
+    const int set = DIST == 2 ? q : 0;
+#pragma unroll
+    for (int i = 0; i < NPT; ++i)
+      if (has_piece) *(u4*)(xt + q * BUFH + piece_lds[i]) = xg[set][i];
+    if (has_sum) s_xs[q * 2 * ROWS + tid] = xsg[set];
   };
-  for (int i = tid; i < ROWH / 2; i += WG_THREADS) {               // zero rows of both buffers
-    ((uint32_t*)(xt + (size_t)M * ROWH))[i] = 0u;
-    ((uint32_t*)(xt + bufh + (size_t)M * ROWH))[i] = 0u;
-  }
+  if (tid < ROWS) s_sc[tid] = tid < M ? t.sc_g[tid] : 0.f;
   stage_load(c_begin, 0);
-  stage_load(c_begin + 1, 1);
+  if constexpr (DIST == 2) stage_load(c_begin + 1, 1);
 
   // row constants of the output side (scale, sign, bias of rows lane and lane + 64), requested ahead of the weight stream by the workgroup
   // that will finish the row block, so that they have long arrived when it needs them
@@ -1030,65 +1045,84 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear_batch(const uint32_t* __r
 #pragma unroll
   for (int p = 0; p < P; ++p) prefetch(buf[p]);
 
-  // ---- per-lane constants of the product: this lane's B operands and sums belong to activation row 16 mg + lane % 16
-  int boff[MG], xsoff[MG];
-  float sc[MG], offs[MG], k1534[MG];
-#pragma unroll
-  for (int mg = 0; mg < MG; ++mg) {
-    const int mrow = mg * 16 + n16;
-    const bool live = mrow < M;
-    boff[mg] = (live ? mrow : M) * ROWH + 8 * (4 * ch + g);
-    xsoff[mg] = live ? 2 * mrow + ch : 0;
-    offs[mg] = 0.f;
-    sc[mg] = live ? t.sc_g[mrow] : 0.f;
-    k1534[mg] = live ? 1534.f : 0.f;
-  }
+  // ---- the product.  This lane's B operands and sums belong to activation rows 16 mg + lane % 16: group mg sits
+  // 16 mg rows behind group 0 in LDS, a constant offset
+  const _Float16* b_lane = xt + n16 * ROWH + 8 * (4 * ch + g);
+  const float* xs_lane = s_xs + 2 * n16 + ch;
+  float offs[MG];      // running 1534 * sum(x~) over the wave's half of the blocks
   f4 acc[MG][2];
 #pragma unroll
-  for (int mg = 0; mg < MG; ++mg) { acc[mg][0] = f4{0.f, 0.f, 0.f, 0.f}; acc[mg][1] = f4{0.f, 0.f, 0.f, 0.f}; }
+  for (int mg = 0; mg < MG; ++mg) { offs[mg] = 0.f; acc[mg][0] = f4{0.f, 0.f, 0.f, 0.f}; acc[mg][1] = f4{0.f, 0.f, 0.f, 0.f}; }
 
-  h8 B0[MG], B1[MG];
-  float xsv[MG];
+  // B operands and sums: up to 32 rows they are read one step ahead, right behind the barrier, and their latency hides
+  // behind the second half of the decode; with more rows they would hold too many registers, and each pair of 16-row
+  // groups is read while the matrix instructions of the pair before it run
+  constexpr bool AHEAD = MG <= 2;
+  constexpr int NB = AHEAD ? MG : 4;               // B register sets
+  h8 B0[NB], B1[NB];
+  float xsv[NB];
+  auto fetch_b = [&](int bsel, int mg, int set) {
+    const _Float16* bp = b_lane + bsel * BUFH + mg * 16 * ROWH;
+    B0[set] = *(const h8*)bp;
+    B1[set] = *(const h8*)(bp + 64);
+    xsv[set] = xs_lane[bsel * 2 * ROWS + mg * 32];
+  };
   auto load_b = [&](int bsel) {
+    if constexpr (AHEAD) {
 #pragma unroll
-    for (int mg = 0; mg < MG; ++mg) {
-      const _Float16* bp = xt + bsel * bufh + boff[mg];
-      B0[mg] = *(const h8*)bp;
-      B1[mg] = *(const h8*)(bp + 64);
-      xsv[mg] = s_xs[bsel * 2 * M + xsoff[mg]];
+      for (int mg = 0; mg < MG; ++mg) fetch_b(bsel, mg, mg);
+    }
+  };
+  auto multiply = [&](const DecodedStep<K>& d, int bsel) {
+    if constexpr (AHEAD) {
+#pragma unroll
+      for (int mg = 0; mg < MG; ++mg) acc[mg][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[0], B0[mg], acc[mg][0], 0, 0, 0);
+#pragma unroll
+      for (int mg = 0; mg < MG; ++mg) acc[mg][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[2], B0[mg], acc[mg][1], 0, 0, 0);
+#pragma unroll
+      for (int mg = 0; mg < MG; ++mg) acc[mg][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[1], B1[mg], acc[mg][0], 0, 0, 0);
+#pragma unroll
+      for (int mg = 0; mg < MG; ++mg) acc[mg][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[3], B1[mg], acc[mg][1], 0, 0, 0);
+#pragma unroll
+      for (int mg = 0; mg < MG; ++mg) offs[mg] = __builtin_fmaf(1534.f, xsv[mg], offs[mg]);
+    } else {
+      fetch_b(bsel, 0, 0); fetch_b(bsel, 1, 1);
+#pragma unroll
+      for (int pr = 0; pr < MG / 2; ++pr) {
+        const int cs = (pr & 1) * 2;
+        if (pr + 1 < MG / 2) { fetch_b(bsel, 2 * pr + 2, cs ^ 2); fetch_b(bsel, 2 * pr + 3, (cs ^ 2) + 1); }
+#pragma unroll
+        for (int u = 0; u < 2; ++u) acc[2 * pr + u][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[0], B0[cs + u], acc[2 * pr + u][0], 0, 0, 0);
+#pragma unroll
+        for (int u = 0; u < 2; ++u) acc[2 * pr + u][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[2], B0[cs + u], acc[2 * pr + u][1], 0, 0, 0);
+#pragma unroll
+        for (int u = 0; u < 2; ++u) acc[2 * pr + u][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[1], B1[cs + u], acc[2 * pr + u][0], 0, 0, 0);
+#pragma unroll
+        for (int u = 0; u < 2; ++u) acc[2 * pr + u][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[3], B1[cs + u], acc[2 * pr + u][1], 0, 0, 0);
+#pragma unroll
+        for (int u = 0; u < 2; ++u) offs[2 * pr + u] = __builtin_fmaf(1534.f, xsv[cs + u], offs[2 * pr + u]);
+      }
     }
   };
 
-  // step 0: its block goes to buffer 0, the block of step 2 is requested, the first weights are decoded meanwhile
+  // step 0: its block goes to buffer 0, the next block to come is requested, the first weights are decoded meanwhile
   static_assert(P % 2 == 0, "the block parity of a step must be static in the unrolled loop");
   const int hist = history_lane_byteaddr(lane);
   stage_store(0);
-  stage_load(c_begin + 2, 0);
+  stage_load(c_begin + DIST, 0);
   DecodedStep<K> cur;
   decode_step<K>(buf[0], hist, cur);
   prefetch(buf[0]);
   __syncthreads();
   load_b(0);
 
-  auto multiply = [&](const DecodedStep<K>& d) {
-#pragma unroll
-    for (int mg = 0; mg < MG; ++mg) acc[mg][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[0], B0[mg], acc[mg][0], 0, 0, 0);
-#pragma unroll
-    for (int mg = 0; mg < MG; ++mg) acc[mg][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[2], B0[mg], acc[mg][1], 0, 0, 0);
-#pragma unroll
-    for (int mg = 0; mg < MG; ++mg) acc[mg][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[1], B1[mg], acc[mg][0], 0, 0, 0);
-#pragma unroll
-    for (int mg = 0; mg < MG; ++mg) acc[mg][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[3], B1[mg], acc[mg][1], 0, 0, 0);
-#pragma unroll
-    for (int mg = 0; mg < MG; ++mg) offs[mg] = __builtin_fmaf(k1534[mg], xsv[mg], offs[mg]);
-  };
-  // One step with a successor: multiply step v, put the block of step v + 1 (in registers since the previous step)
-  // into the other buffer, request the block of step v + 2, decode step v + 1; between the two halves of the decode
-  // the workgroup meets, after which the B operands of step v + 1 are read (their latency hides behind the rest).
+  // One step with a successor: multiply step v, put the block of step v + 1 (in registers) into the other buffer,
+  // request the next block to come, decode step v + 1; between the two halves of the decode the workgroup meets, after
+  // which the B operands of step v + 1 may be read.
   auto step_with_next = [&](int v, int q, StreamRegs<K>& nxt) {      // q = (v + 1) & 1, static
-    multiply(cur);
+    multiply(cur, q ^ 1);
     stage_store(q);
-    stage_load(c_begin + v + 3, q);
+    stage_load(c_begin + v + 1 + DIST, q);
     decode_step_mid<K>(nxt, hist, cur, [&]() { __syncthreads(); load_b(q); });
     prefetch(nxt);
   };
@@ -1100,10 +1134,14 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear_batch(const uint32_t* __r
 #pragma unroll
   for (int pp = 0; pp < P; ++pp) {
     if (v + pp + 1 < nsteps) step_with_next(v + pp, (pp + 1) & 1, buf[(pp + 1) % P]);
-    else if (v + pp < nsteps) multiply(cur);
+    else if (v + pp < nsteps) multiply(cur, pp & 1);
   }
 
   // ---- this wave's partial (offset removed, activation scale undone) goes to its column half's copy in LDS
+  float scl[MG];
+#pragma unroll
+  for (int mg = 0; mg < MG; ++mg) scl[mg] = s_sc[mg * 16 + n16];
+  if constexpr (FIN_OVER_BLOCKS) __syncthreads();          // every wave has read its last B operands
 #pragma unroll
   for (int mg = 0; mg < MG; ++mg) {
     const int mrow = mg * 16 + n16;
@@ -1113,7 +1151,7 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear_batch(const uint32_t* __r
       for (int j = 0; j < 4; ++j)
 #pragma unroll
         for (int rr = 0; rr < 2; ++rr)
-          dst[(2 * j + rr) * 16] = (acc[mg][rr][j] - offs[mg]) * sc[mg];
+          dst[(2 * j + rr) * 16] = (acc[mg][rr][j] - offs[mg]) * scl[mg];
     }
   }
   __syncthreads();
@@ -1196,37 +1234,44 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear_batch(const uint32_t* __r
   // repeats the last slot).
   auto finish_rows_together = [&](auto jw) {
     constexpr int JW = decltype(jw)::value;
-    float a0[RPW], a1[RPW];
-    int tries = 0;
-    bool failed = false;
-    for (;;) {
-      uint32_t u0[RPW][JW], u1[RPW][JW];
+    constexpr int RB = RPW * JW <= 32 ? RPW : 32 / JW;      // rows per request: at most 2 x 32 registers of slots
 #pragma unroll
-      for (int r = 0; r < RPW; ++r)
+    for (int rbase = 0; rbase < RPW; rbase += RB) {
+      if (w + rbase * WG_WAVES >= M) break;
+      float a0[RB], a1[RB];
+      int tries = 0;
+      bool failed = false;
+      for (;;) {
+        uint32_t u0[RB][JW], u1[RB][JW];
 #pragma unroll
-        for (int k = 0; k < JW; ++k) {
-          const uint32_t* pp = slot_of(min(k, S - 2), min(w + r * WG_WAVES, M - 1));
-          u0[r][k] = __hip_atomic_load(pp + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          u1[r][k] = __hip_atomic_load(pp + lane + 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-      bool missing = false;
+        for (int r = 0; r < RB; ++r)
 #pragma unroll
-      for (int r = 0; r < RPW; ++r) {
-        a0[r] = 0.f; a1[r] = 0.f;
-#pragma unroll
-        for (int k = 0; k < JW; ++k)
-          if (k < S - 1) {
-            missing |= (u0[r][k] == 0u) | (u1[r][k] == 0u);
-            a0[r] += __uint_as_float(u0[r][k]); a1[r] += __uint_as_float(u1[r][k]);
+          for (int k = 0; k < JW; ++k) {
+            const uint32_t* pp = slot_of(min(k, S - 2), min(w + (rbase + r) * WG_WAVES, M - 1));
+            u0[r][k] = __hip_atomic_load(pp + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            u1[r][k] = __hip_atomic_load(pp + lane + 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           }
-      }
-      if (!__any(missing)) break;
-      if (++tries >= t.spin_limit) { failed = true; break; }
-      __builtin_amdgcn_s_sleep(2);
-    }
+        bool missing = false;
 #pragma unroll
-    for (int r = 0; r < RPW; ++r)
-      if (w + r * WG_WAVES < M) finish_row(w + r * WG_WAVES, a0[r], a1[r], failed);
+        for (int r = 0; r < RB; ++r) {
+          a0[r] = 0.f; a1[r] = 0.f;
+          // a row beyond M repeats the request of row M - 1, whose own wave may have cleared its slots already: not waited for
+          const bool real = w + (rbase + r) * WG_WAVES < M;
+#pragma unroll
+          for (int k = 0; k < JW; ++k)
+            if (real && k < S - 1) {
+              missing |= (u0[r][k] == 0u) | (u1[r][k] == 0u);
+              a0[r] += __uint_as_float(u0[r][k]); a1[r] += __uint_as_float(u1[r][k]);
+            }
+        }
+        if (!__any(missing)) break;
+        if (++tries >= t.spin_limit) { failed = true; break; }
+        __builtin_amdgcn_s_sleep(2);
+      }
+#pragma unroll
+      for (int r = 0; r < RB; ++r)
+        if (w + (rbase + r) * WG_WAVES < M) finish_row(w + (rbase + r) * WG_WAVES, a0[r], a1[r], failed);
+    }
   };
   if (S > 1 && S - 1 <= 8 && w + WG_WAVES < M) {
     if (S - 1 <= 1) finish_rows_together(std::integral_constant<int, 1>{});
@@ -1703,10 +1748,15 @@ template <int K> int launch_linear_k(const LinearLaunch& a, bool prerot, int mb,
 // ---- batched kernel: split S of the column blocks per row block
 struct BatchPlan { int S, cb, wgs, mb; size_t lds; };
 constexpr int BATCH_MIN_M = 6;      // rows from which the library policy takes the batched kernel
-inline size_t batch_lds_bytes(int M) { return (size_t)2 * (M + 1) * BATCH_ROWH * 2 + (size_t)4 * M * 4 + (size_t)2 * M * BATCH_FIN_STRIDE * 4; }
+inline int batch_groups(int M) { return M <= 16 ? 1 : (M <= 32 ? 2 : (M <= 64 ? 4 : 8)); }   // groups of 16 activation rows
+inline size_t batch_lds_bytes(int M) {
+  const int rows = 16 * batch_groups(M);
+  const size_t blocks = (size_t)2 * rows * BATCH_ROWH * 2, small = (size_t)5 * rows * 4, fin = (size_t)2 * M * BATCH_FIN_STRIDE * 4;
+  return M > 64 ? (blocks + small > fin ? blocks + small : fin) : blocks + small + fin;
+}
 inline bool make_batch_plan(int m, int n, int M, int want_S, BatchPlan& bp) {
   const int nblk = n / 128, rbs = m / 128;
-  bp.mb = M <= 16 ? 1 : 2;                  // groups of 16 activation rows
+  bp.mb = batch_groups(M);
   bp.lds = batch_lds_bytes(M);
   // Measured on MI355X (K4, 8..32 rows, 4096..28672 output rows): one workgroup per CU is the best fill; every further
   // split adds partial traffic that grows with the rows.  So: the largest split that keeps the grid within the CU
@@ -1744,7 +1794,9 @@ template <int K> int launch_batch_k(const uint32_t* qw, float* part, int m, int 
                                     const BatchPlan& bp, hipStream_t st) {
   switch (bp.mb) {
     case 1: return launch_batch_v<K, 1>(qw, part, m, n, M, flags, t, bp, st);
-    default: return launch_batch_v<K, 2>(qw, part, m, n, M, flags, t, bp, st);
+    case 2: return launch_batch_v<K, 2>(qw, part, m, n, M, flags, t, bp, st);
+    case 4: return launch_batch_v<K, 4>(qw, part, m, n, M, flags, t, bp, st);
+    default: return launch_batch_v<K, 8>(qw, part, m, n, M, flags, t, bp, st);
   }
 }
 // nsplit bit 29: batched kernel with the split in the low bits (0 = policy); otherwise the policy decides by M
@@ -1797,6 +1849,7 @@ size_t htr_workspace_bytes(int m, int n, int K, int M, int nsplit) {
     if (!make_batch_plan(m, n, M, nsplit > 0 ? nsplit & 0xFFFFF : 0, bp)) return 0;
     return ws_need((size_t)bp.wgs * M * 128 * sizeof(float), prerot_bytes(n, M));
   }
+  if (M > HTR_MAX_GROUP_ROWS) return 0;          // the chunked kernel takes up to 32 rows
   Plan pl;
   if (!make_plan(m, n, M, nsplit, pl)) return 0;
   return ws_need((size_t)pl.wgs * M * 128 * sizeof(float), prerot_bytes(n, M));
@@ -1813,6 +1866,7 @@ int htr_linear_plan(int m, int n, int K, int M, int nsplit, int* out6) {
     out6[0] = bp.cb; out6[1] = bp.wgs; out6[2] = 1; out6[3] = 1; out6[4] = 1; out6[5] = (int)bp.lds;
     return HTR_OK;
   }
+  if (M > HTR_MAX_GROUP_ROWS) return HTR_ERR_BATCH;
   Plan pl;
   if (!make_plan(m, n, M, nsplit, pl)) return HTR_ERR_SPLIT;
   out6[0] = pl.chunk; out6[1] = pl.wgs; out6[2] = pl.segfin; out6[3] = pl.nbl; out6[4] = pl.prerot; out6[5] = (int)pl.lds;
@@ -1858,6 +1912,7 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
     HTR_FOR_K(K, return launch_batch_k<KK>((const uint32_t*)qweight, part, m, n, M, flags, t, bp, st));
     return HTR_OK;
   }
+  if (M > HTR_MAX_GROUP_ROWS) return HTR_ERR_BATCH;          // an explicit chunked plan: that kernel takes up to 32 rows
   Plan pl;
   if (!make_plan(m, n, M, nsplit, pl)) return HTR_ERR_SPLIT;
   // the in-kernel rotation reads 16-bit elements in pairs: float32 activations, and rows that do not start on a
@@ -1928,7 +1983,7 @@ static bool make_group_plan(int count, int m, int n, int max_M, Plan& pl) {
 }
 
 size_t htr_grouped_workspace_bytes(int count, int m, int n, int K, int max_M) {
-  if (K < 2 || K > 8 || !shape_ok(m, n) || max_M < 1 || max_M > HTR_MAX_BATCH || count < 1 || count > HTR_MAX_GROUP) return 0;
+  if (K < 2 || K > 8 || !shape_ok(m, n) || max_M < 1 || max_M > HTR_MAX_GROUP_ROWS || count < 1 || count > HTR_MAX_GROUP) return 0;
   Plan pl;
   if (!make_group_plan(count, m, n, max_M, pl)) return 0;
   return ws_need((size_t)count * pl.wgs * max_M * 128 * sizeof(float), (size_t)count * prerot_bytes(n, max_M));
@@ -1940,7 +1995,7 @@ int htr_linear_grouped(const htr_group_entry* entries, int count, int m, int n, 
   if (count < 1 || count > HTR_MAX_GROUP) return HTR_ERR_COUNT;
   if (K < 2 || K > 8) return HTR_ERR_K;
   if (!shape_ok(m, n)) return HTR_ERR_SHAPE;
-  if (max_M < 1 || max_M > HTR_MAX_BATCH) return HTR_ERR_BATCH;
+  if (max_M < 1 || max_M > HTR_MAX_GROUP_ROWS) return HTR_ERR_BATCH;
   if (!dtype_ok(x_dtype) || !dtype_ok(y_dtype)) return HTR_ERR_DTYPE;
   if ((uintptr_t)entries & 7) return HTR_ERR_ALIGN;
   Plan pl;

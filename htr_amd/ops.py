@@ -17,14 +17,15 @@ _DTYPE_CODE = {torch.bfloat16: _native.BF16, torch.float16: _native.F16, torch.f
 # One launch takes up to this many activation rows; longer inputs are cut into chunks that each
 # re-read the packed weight (the reference does the same in 8-row chunks, htr/ops.py:77-88).
 LAUNCH_MAX_M = _native.MAX_BATCH
+GROUP_MAX_M = _native.MAX_GROUP_ROWS      # rows per entry of a grouped launch
 # explicit chunk length (steps per workgroup) for experiments; 0 = library policy
 NSPLIT = int(os.environ.get("HTR_NSPLIT", "0"))
 # Above this many activation rows the weight is dequantized once to the original basis (bf16) and a library GEMM does
 # the product, as the reference does for prefill (HTR_PREFILL="w", htr/ops.py:52-54,89-93); up to it, the fused
 # decode kernel runs in launches of LAUNCH_MAX_M rows (the reference's HTR_GEMV_LOOP_MAX, htr/ops.py:59-61).
-# Measured on MI355X (K4, eager calls): 32-row fused launches beat dequantize + GEMM up to 40 rows on 4096x4096 and up to
-# about 75 rows on 14336x4096 and 4096x14336.
-GEMV_LOOP_MAX = int(os.environ.get("HTR_GEMV_LOOP_MAX", "64"))
+# Measured on MI355X (K4): one fused launch of 128 rows takes 32 / 42 / 59 us on 4096x4096 / 14336x4096 / 4096x14336,
+# dequantize + GEMM 42 / 73 / 105 us; two fused launches (256 rows) no longer beat it.
+GEMV_LOOP_MAX = int(os.environ.get("HTR_GEMV_LOOP_MAX", "128"))
 
 _WORKSPACES = {}
 
@@ -101,7 +102,7 @@ def linear_grouped(xs, weights, biases=None, out_dtype=None):
     xs: list of [M_i, n] tensors (M_i may be 0); weights: list of (qweight, scales, su, sv) of identical shapes and K;
     returns the list of [M_i, m] results.  Routed experts are the use: the reference has no kernel for them and runs
     one linear per expert (docs/ADAPTERS.md:19 of the reference), which on this GPU is dominated by launch latency.
-    Problems with more than LAUNCH_MAX_M rows are cut into several table entries.
+    Problems with more than GROUP_MAX_M rows are cut into several table entries.
     """
     if len(xs) != len(weights) or not xs:
         raise RuntimeError("linear_grouped wants as many activation tensors as weight tuples, at least one")
@@ -132,8 +133,8 @@ def linear_grouped(xs, weights, biases=None, out_dtype=None):
         xc = x.contiguous()
         keep.append(xc)
         outs.append(y[r:r + rows[i]])
-        for r0 in range(0, rows[i], LAUNCH_MAX_M):
-            mi = min(LAUNCH_MAX_M, rows[i] - r0)
+        for r0 in range(0, rows[i], GROUP_MAX_M):
+            mi = min(GROUP_MAX_M, rows[i] - r0)
             entries.append([w[0].data_ptr(), w[1].data_ptr(), w[2].data_ptr(), w[3].data_ptr(),
                             xc[r0:r0 + mi].data_ptr(), 0 if b is None else b.data_ptr(), y[r + r0:r + r0 + mi].data_ptr(), mi])
         r += rows[i]

@@ -43,7 +43,8 @@ typedef enum {
 /* element type codes; same numbering as the reference's out-dtype map (htr/ops.py:79,94) */
 enum { HTR_BF16 = 0, HTR_F16 = 1, HTR_F32 = 2 };
 
-#define HTR_MAX_BATCH 32   /* activation rows one htr_linear launch accepts */
+#define HTR_MAX_BATCH 128       /* activation rows one htr_linear launch accepts */
+#define HTR_MAX_GROUP_ROWS 32   /* rows per problem of htr_linear_grouped (and of an explicit chunked plan, see nsplit) */
 #define HTR_MAX_GROUP 4096 /* problems one htr_linear_grouped launch accepts */
 
 const char* htr_strerror(int status);
@@ -118,7 +119,7 @@ typedef struct {
  * decode-product-epilogue for all problems): routed experts, whose per-expert launches would each pay the full launch
  * latency for a few microseconds of work.  No counterpart in the reference, which has no runtime kernel for routed
  * experts and composes them from per-expert linears (docs/ADAPTERS.md:19); the per-problem result is that of
- * htr_linear on the same tensors.  max_M bounds the rows of any problem (1 .. HTR_MAX_BATCH).
+ * htr_linear on the same tensors.  max_M bounds the rows of any problem (1 .. HTR_MAX_GROUP_ROWS).
  * Workspace: htr_grouped_workspace_bytes() bytes, zeroed once, same rules as for htr_linear.
  */
 size_t htr_grouped_workspace_bytes(int count, int m, int n, int K, int max_M);

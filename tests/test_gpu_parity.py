@@ -120,7 +120,8 @@ def test_linear_f32_out_within_tolerance(dev, oracle, K, M, shape):
     assert _rel(y, ref) <= REL_TOL, _rel(y, ref)
 
 
-@pytest.mark.parametrize("K,M", [(3, 16), (4, 9), (4, 16), (4, 32), (3, 32), (5, 17), (4, 45), (4, 100), (2, 8), (8, 24)])
+@pytest.mark.parametrize("K,M", [(3, 16), (4, 9), (4, 16), (4, 32), (3, 32), (5, 17), (4, 45), (4, 100), (2, 8), (8, 24), (4, 6), (4, 7), (4, 64),
+                                 (3, 50), (5, 33), (6, 64), (2, 49), (7, 40), (8, 64), (4, 65), (4, 128), (3, 97), (8, 128), (5, 111)])
 def test_linear_small_batch_blocks(dev, oracle, K, M, monkeypatch):
     from htr_amd import ops
     print(f"linear batch K={K} M={M}", flush=True)
@@ -251,10 +252,12 @@ def test_full_size_shapes(dev, oracle, K, m, n):
 
 # ---- the small-batch GEMM shapes, the 64-expert stack and the output head as parity cases
 @pytest.mark.parametrize("K,M,m,n", [(3, 8, 14336, 4096), (4, 16, 14336, 4096), (4, 32, 4096, 14336), (3, 32, 14336, 4096),
-                                     (4, 8, 4096, 14336)])
-def test_small_batch_gemm_shapes(dev, oracle, K, M, m, n):
+                                     (4, 8, 4096, 14336), (4, 64, 14336, 4096), (4, 48, 4096, 14336), (4, 6, 4096, 4096),
+                                     (4, 128, 4096, 4096), (4, 100, 14336, 4096)])
+def test_small_batch_gemm_shapes(dev, oracle, K, M, m, n, monkeypatch):
     from htr_amd import ops
     print(f"small-batch K={K} M={M} {m}x{n}", flush=True)
+    monkeypatch.setattr(ops, "GEMV_LOOP_MAX", 1 << 30)     # the fused kernel at every M
     qw, sc, su, sv, x = _case(m, n, K, M, 4000 + 13 * K + M)
     y = ops.linear_f32out(x.to(dev), *[t.to(dev) for t in (qw, sc, su, sv)]).cpu().numpy()
     ref = _ref(oracle, qw, sc, su, sv, x)
@@ -369,18 +372,19 @@ def test_lm_head_shape(dev, oracle):
     assert _rel(y, ref) <= REL_TOL, _rel(y, ref)
 
 
-def test_seeded_sweep_of_shapes_rows_and_widths(dev, oracle):
+def test_seeded_sweep_of_shapes_rows_and_widths(dev, oracle, monkeypatch):
     """Forty-eight seeded combinations of output and input size (multiples of 128 up to 2048, so every chunking case
     of the planner: aligned, ragged, chunks across row blocks, a single workgroup), bit width, row count (all three
     kernels: chunked, batched, fused-launch loop), activation type and bias, each against the float64 oracle."""
     from htr_amd import ops
+    monkeypatch.setattr(ops, "GEMV_LOOP_MAX", 1 << 30)     # the fused kernels at every M
     rng = np.random.default_rng(20261125)
     worst = 0.0
     for case in range(48):
         m = int(rng.integers(1, 17)) * 128
         n = int(rng.integers(1, 17)) * 128
         K = int(rng.choice([2, 3, 4, 5, 6, 7, 8]))
-        M = int(rng.choice([1, 1, 1, 2, 3, 4, 5, 7, 8, 9, 15, 16, 17, 31, 32, 33, 40]))
+        M = int(rng.choice([1, 1, 1, 2, 3, 4, 5, 6, 7, 8, 9, 15, 16, 17, 31, 32, 33, 40, 48, 63, 64, 65, 96, 127, 128]))
         dtype = [torch.bfloat16, torch.float16, torch.float32][int(rng.integers(0, 3))]
         with_bias = bool(rng.integers(0, 2))
         print(f"sweep case {case}: {m}x{n} K={K} M={M} {dtype} bias={with_bias}", flush=True)

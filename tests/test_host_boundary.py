@@ -52,7 +52,8 @@ def test_validation_codes_without_gpu(L):
     assert call(qw=None) == 1
     assert call(K=1) == 2 and call(K=9) == 2
     assert call(m=200) == 3 and call(n=0) == 3
-    assert call(M=0) == 4 and call(M=33) == 4
+    assert call(M=0) == 4 and call(M=129) == 4
+    assert call(M=33, ns=4) == 4               # an explicit chunked plan stops at 32 rows
     assert call(xd=3) == 5 and call(yd=-1) == 5
     assert call(ws=None) == 6 and call(wsb=16) == 6 and call(ws=ctypes.c_void_p(0x100010)) == 6
     assert call(qw=ctypes.c_void_p(0x1004)) == 7
@@ -64,7 +65,7 @@ def test_validation_codes_without_gpu(L):
 
 @pytest.mark.parametrize("m,n", [(128, 128), (256, 384), (4096, 4096), (1024, 4096), (6144, 4096), (14336, 4096),
                                  (28672, 4096), (4096, 14336), (152064, 4096), (1408, 2048), (2048, 1408)])
-@pytest.mark.parametrize("M", [1, 2, 8, 9, 16, 32])
+@pytest.mark.parametrize("M", [1, 2, 5, 6, 8, 9, 16, 32, 33, 64, 65, 128])
 def test_launch_plan_is_consistent(L, m, n, M):
     out = (ctypes.c_int * 6)()
     assert L.htr_linear_plan(m, n, 4, M, 0, out) == 0
@@ -72,11 +73,11 @@ def test_launch_plan_is_consistent(L, m, n, M):
     nblk, rbs = n // 128, m // 128
     need = L.htr_workspace_bytes(m, n, 4, M, 0)
     assert need >= 256 + wgs * M * 128 * 4                                       # header + one partial slot per workgroup
-    if M >= 8:
+    if M >= 6:
         # batched kernel: `chunk` column blocks per split, S = ceil(nblk / chunk) splits per row block, no empty split,
         # activations always rotated ahead
         S = -(-nblk // chunk)
-        assert wgs == rbs * S and (S - 1) * chunk < nblk and prerot == 1 and lds <= 64 * 1024
+        assert wgs == rbs * S and (S - 1) * chunk < nblk and prerot == 1 and lds <= (64 if M <= 32 else 140) * 1024
         # an explicit split is honoured (bit 29 selects the batched kernel)
         assert L.htr_linear_plan(m, n, 4, M, (1 << 29) | 1, out) == 0 and out[0] == nblk and out[1] == rbs
         return

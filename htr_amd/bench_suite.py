@@ -1,5 +1,5 @@
 """Timings of the packed-linear path beyond the headline layer: the other configurations the reference's baseline
-names (K x shape x batch table, 8..32 activation rows, routed experts, lm_head) and the prefill path.
+names (K x shape x batch table, 8..128 activation rows, routed experts, lm_head) and the prefill path.
 
 Every case cycles through a ring of distinct weight copies larger than the caches (>= 1 GB, or as many copies as
 fit), replays the ring as one HIP graph and reads HIP events on the launch stream.  Used by `bench.py --suite`;
@@ -78,10 +78,10 @@ def table(dev):
 
 
 def batch(dev):
-    """K3, K4 x 8, 16, 32 activation rows x {14336x4096, 4096x14336}; also the rate in TFLOP/s (2 M m n)."""
+    """K3, K4 x 8 .. 128 activation rows x {14336x4096, 4096x14336}; also the rate in TFLOP/s (2 M m n)."""
     out = []
     for K in (3, 4):
-        for M in (8, 16, 32):
+        for M in (8, 16, 32, 64, 128):
             for (m, n) in ((14336, 4096), (4096, 14336)):
                 r = time_linear(m, n, K, M, dev)
                 r["TFLOPs"] = round(2.0 * M * m * n / r["us"] / 1e6, 1)

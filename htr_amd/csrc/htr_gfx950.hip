@@ -1758,11 +1758,12 @@ inline bool make_batch_plan(int m, int n, int M, int want_S, BatchPlan& bp) {
   const int nblk = n / 128, rbs = m / 128;
   bp.mb = batch_groups(M);
   bp.lds = batch_lds_bytes(M);
-  // Measured on MI355X (K4, 8..32 rows, 4096..28672 output rows): one workgroup per CU is the best fill; every further
-  // split adds partial traffic that grows with the rows.  So: the largest split that keeps the grid within the CU
-  // count, among the splits that leave no column range empty.
-  // Splits shorter than 8 column blocks cost more in partial traffic and set-up than their parallelism returns
-  // (4096x4096, 16 and 32 rows: 4 splits of 8 blocks beat 8 of 4 by 5..8 %), unless fewer than half the CUs would have work.
+  // Measured on MI355X (K4, 6..128 rows, 4096..28672 output rows): one workgroup per CU is the best fill; every further
+  // split adds partial traffic that grows with the rows (14336x4096, 32 rows: 2 splits 20.3 us, 4 splits 25.8; 128
+  // rows: 43 against 62).  So: the largest split that keeps the grid within the CU count, among the splits that leave
+  // no column range empty.  Splits shorter than 8 column blocks cost more in partial traffic and set-up than their
+  // parallelism returns (4096x4096, 32 rows: 4 splits of 8 blocks 14.8 us, 8 of 4 16.7; 128 rows: 31.7 against 41.4),
+  // unless fewer than half the CUs would have work.
   const int limit = want_S > 0 ? want_S : (NUM_CU / rbs > 1 ? NUM_CU / rbs : 1);
   bool found = false, found_long = false;
   BatchPlan longer = bp;

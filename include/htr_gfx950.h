@@ -78,7 +78,11 @@ size_t htr_workspace_bytes(int m, int n, int K, int M, int nsplit);
  * per workgroup, workgroups, row blocks that can end inside one workgroup's chunk, distinct column blocks per
  * workgroup, 1 if the activations are rotated by a launch of their own, dynamic LDS bytes}.  No reference counterpart
  * as a function; it exposes what nsplit_for / fused_nsplit decide there (htr/ops.py:31-45).
- * nsplit: 0 = library policy; otherwise the steps per workgroup (bit 30 set: force the separate rotation launch).
+ * With 6 rows and more (library policy) the batched kernel runs instead: out6 = {column blocks per split, workgroups
+ * (= row blocks x splits), 1, 1, 1, dynamic LDS bytes}.
+ * nsplit: 0 = library policy; otherwise the steps per workgroup of the chunked kernel (1 .. HTR_MAX_GROUP_ROWS rows;
+ * bit 30 set: force the separate rotation launch), or, with bit 29 set, the batched kernel with that many column
+ * splits in the low bits (0 = its own policy).
  */
 int htr_linear_plan(int m, int n, int K, int M, int nsplit, int* out6);
 
@@ -87,7 +91,7 @@ int htr_linear_plan(int m, int n, int K, int M, int nsplit, int* out6);
  * H128, trellis decode, row scale, fp32-accumulated product, output H128 + sign, bias, cast.
  * Reference: the decode branch of _linear_impl (htr/ops.py:75-76, :94-98), i.e.
  * prologue + gemv_epi / gemv_fused (htr/csrc/htr_kernels.cu:972-987, :1134-1173, :1034-1064).
- *   x      [M, n] row-major, x_dtype (bf16 / f16 / f32)
+ *   x      [M, n] row-major, x_dtype (bf16 / f16 / f32), 1 <= M <= HTR_MAX_BATCH
  *   bias   [m] in y_dtype, or NULL
  *   y      [M, m] row-major, y_dtype
  *   nsplit 0 = library policy; otherwise an explicit plan as in htr_linear_plan (tuning)

@@ -1006,9 +1006,11 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear_batch(const uint32_t* __r
   stage_load(c_begin, 0);
   if constexpr (DIST == 2) stage_load(c_begin + 1, 1);
 
-  // row constants of the output side (scale, sign, bias of rows lane and lane + 64), requested ahead of the weight stream by the workgroup
-  // that will finish the row block, so that they have long arrived when it needs them
-  const bool finisher = s_idx == S - 1;
+  // row constants of the output side (scale, sign, bias of rows lane and lane + 64), requested ahead of the weight stream by
+  // the workgroups that finish rows of the row block, so that they have long arrived when they are needed
+  const int RG = (M + 7) >> 3;               // groups of eight activation rows
+  const bool spread = M > 16;                // the splits share the output side (below)
+  const bool finisher = spread ? s_idx < RG : s_idx == S - 1;
   const int r0 = rb * 128 + lane, r1 = r0 + 64;
   uint32_t raw_sc0 = 0u, raw_sc1 = 0u, raw_sv0 = 0u, raw_sv1 = 0u, raw_b0 = 0u, raw_b1 = 0u;   // bits only: converted at the end
   if (finisher) {
@@ -1156,18 +1158,26 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear_batch(const uint32_t* __r
   }
   __syncthreads();
   const int pos0 = batch_fin_pos(lane), pos1 = batch_fin_pos(lane + 64);
-  if (!finisher) {
-    for (int mrow = w; mrow < M; mrow += WG_WAVES) {
+  // ---- exchange between the splits of the row block.  The activation rows are dealt to the splits in groups of eight
+  // (group rg = rows 8 rg .. 8 rg + 7, one row per wave): split rg mod S finishes group rg, every other split leaves
+  // its partial of those rows in its slot.  So the output side of many rows is spread over the splits instead of
+  // falling to one workgroup (32 rows on 4096x14336, 8 splits: 23.0 -> 19.7 us; 128 rows: 56.6 -> 38.5).  The
+  // workgroups of one row block are neighbours in dispatch order and the grid fits the chip, so they run together; the
+  // wait is bounded all the same.  Up to 16 rows the last split finishes everything, as in k_linear: two workgroups
+  // that wait for each other cost 0.3 us more than one that waits.
+  for (int rg = 0, owner = spread ? 0 : S - 1; rg < RG; ++rg, owner = !spread ? owner : (owner + 1 == S ? 0 : owner + 1)) {
+    const int mrow = 8 * rg + w;
+    if (owner != s_idx && mrow < M) {
       const float* own = s_fin + mrow * BATCH_FIN_STRIDE;
       const float* oth = own + M * BATCH_FIN_STRIDE;
       uint32_t* dst = (uint32_t*)(part + (((size_t)rb * S + s_idx) * M + mrow) * 128);
       __hip_atomic_store(dst + lane, __float_as_uint(own[pos0] + oth[pos0]) | 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       __hip_atomic_store(dst + lane + 64, __float_as_uint(own[pos1] + oth[pos1]) | 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    return;
   }
+  if (!finisher) return;
 
-  // ---- output side: the last split of the row block adds the other splits' partials (fixed order) and finishes
+  // ---- output side of this split's row groups: add the other splits' partials (fixed order), finish
   const float rs0 = f16_bits_to_float((uint16_t)raw_sc0) * t.cbscale * INV_SQRT128;
   const float rs1 = f16_bits_to_float((uint16_t)raw_sc1) * t.cbscale * INV_SQRT128;
   const float sg0 = ((raw_sv0 >> (lane & 7)) & 1u) ? -1.f : 1.f, sg1 = ((raw_sv1 >> (lane & 7)) & 1u) ? -1.f : 1.f;
@@ -1175,7 +1185,8 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear_batch(const uint32_t* __r
     return y_dtype == HTR_F32 ? __uint_as_float(b) : y_dtype == HTR_BF16 ? bf16_bits_to_float((uint16_t)b) : f16_bits_to_float((uint16_t)b);
   };
   const float b0v = cvt_bias(raw_b0), b1v = cvt_bias(raw_b1);
-  auto slot_of = [&](int j, int mrow) { return (uint32_t*)(part + (((size_t)rb * S + j) * M + mrow) * 128); };
+  // slot of the k-th other split (k = 0 .. S - 2, own split skipped) for activation row mrow
+  auto slot_of = [&](int k, int mrow) { return (uint32_t*)(part + (((size_t)rb * S + (k + (k >= s_idx ? 1 : 0))) * M + mrow) * 128); };
   // waits (bounded) until every other split's partial of activation row mrow is there; their sum in fixed order
   auto wait_for_row = [&](int mrow, float& v0s, float& v1s) {
     int tries = 0;
@@ -1206,8 +1217,8 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear_batch(const uint32_t* __r
   auto finish_row = [&](int mrow, float v0s, float v1s, bool failed) {
     if (S > 1) {
       if (!failed) {
-        for (int j = 0; j < S - 1; ++j) {
-          uint32_t* pp = slot_of(j, mrow);
+        for (int k = 0; k < S - 1; ++k) {
+          uint32_t* pp = slot_of(k, mrow);
           __hip_atomic_store(pp + lane, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           __hip_atomic_store(pp + lane + 64, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
@@ -1226,37 +1237,40 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear_batch(const uint32_t* __r
     store_elem_g(t.y, y_dtype, (size_t)mrow * m + r0, v0s);
     store_elem_g(t.y, y_dtype, (size_t)mrow * m + r1, v1s);
   };
-  // Wave w finishes activation rows w, w + 8, ...
-  constexpr int RPW = MG * 16 / WG_WAVES;        // rows per wave at most
-  if (w >= M) return;
-  // With up to eight other splits, all of the wave's rows are polled together, so that the rows behind the first cost
-  // no memory round trip of their own.  JW = slots requested per row (the next power of two from S - 1; the surplus
-  // repeats the last slot).
+  // Wave w finishes row w of this split's groups s_idx, s_idx + S, ...: its i-th row is 8 (s_idx + i S) + w (all groups
+  // if the last split finishes everything).
+  constexpr int RPW = MG * 2;                    // rows per wave at most (a single split finishes all groups)
+  auto my_row = [&](int i) { return spread ? 8 * (s_idx + i * S) + w : 8 * i + w; };
+  // With up to eight other splits the slots of several of the wave's rows are requested together (at most 2 x 32
+  // registers of them), so that the rows behind the first cost no memory round trip of their own.  JW = slots
+  // requested per row (the next power of two from S - 1; the surplus repeats the last slot).
   auto finish_rows_together = [&](auto jw) {
     constexpr int JW = decltype(jw)::value;
-    constexpr int RB = RPW * JW <= 32 ? RPW : 32 / JW;      // rows per request: at most 2 x 32 registers of slots
+    constexpr int RB = RPW * JW <= 32 ? RPW : 32 / JW;      // rows per request
 #pragma unroll
     for (int rbase = 0; rbase < RPW; rbase += RB) {
-      if (w + rbase * WG_WAVES >= M) break;
+      if (my_row(rbase) >= M) break;
       float a0[RB], a1[RB];
       int tries = 0;
       bool failed = false;
       for (;;) {
         uint32_t u0[RB][JW], u1[RB][JW];
 #pragma unroll
-        for (int r = 0; r < RB; ++r)
+        for (int r = 0; r < RB; ++r) {
+          // a row beyond M repeats the request of the batch's first row and is not looked at
+          const int mrow = my_row(rbase + r) < M ? my_row(rbase + r) : my_row(rbase);
 #pragma unroll
           for (int k = 0; k < JW; ++k) {
-            const uint32_t* pp = slot_of(min(k, S - 2), min(w + (rbase + r) * WG_WAVES, M - 1));
+            const uint32_t* pp = slot_of(min(k, S - 2), mrow);
             u0[r][k] = __hip_atomic_load(pp + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             u1[r][k] = __hip_atomic_load(pp + lane + 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           }
+        }
         bool missing = false;
 #pragma unroll
         for (int r = 0; r < RB; ++r) {
           a0[r] = 0.f; a1[r] = 0.f;
-          // a row beyond M repeats the request of row M - 1, whose own wave may have cleared its slots already: not waited for
-          const bool real = w + (rbase + r) * WG_WAVES < M;
+          const bool real = my_row(rbase + r) < M;
 #pragma unroll
           for (int k = 0; k < JW; ++k)
             if (real && k < S - 1) {
@@ -1270,25 +1284,21 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear_batch(const uint32_t* __r
       }
 #pragma unroll
       for (int r = 0; r < RB; ++r)
-        if (w + (rbase + r) * WG_WAVES < M) finish_row(w + (rbase + r) * WG_WAVES, a0[r], a1[r], failed);
+        if (my_row(rbase + r) < M) finish_row(my_row(rbase + r), a0[r], a1[r], failed);
     }
   };
-  if (S > 1 && S - 1 <= 8 && w + WG_WAVES < M) {
+  if (my_row(0) >= M) return;
+  if (S > 1 && S - 1 <= 8 && my_row(1) < M) {
     if (S - 1 <= 1) finish_rows_together(std::integral_constant<int, 1>{});
     else if (S - 1 <= 2) finish_rows_together(std::integral_constant<int, 2>{});
     else if (S - 1 <= 4) finish_rows_together(std::integral_constant<int, 4>{});
     else finish_rows_together(std::integral_constant<int, 8>{});
     return;
   }
-  {
+  for (int i = 0; my_row(i) < M; ++i) {
     float v0s = 0.f, v1s = 0.f;
-    const bool failed = S > 1 ? wait_for_row(w, v0s, v1s) : false;
-    finish_row(w, v0s, v1s, failed);
-  }
-  for (int mrow = w + WG_WAVES; mrow < M; mrow += WG_WAVES) {
-    float v0s = 0.f, v1s = 0.f;
-    const bool failed = S > 1 ? wait_for_row(mrow, v0s, v1s) : false;
-    finish_row(mrow, v0s, v1s, failed);
+    const bool failed = S > 1 ? wait_for_row(my_row(i), v0s, v1s) : false;
+    finish_row(my_row(i), v0s, v1s, failed);
   }
 }
 
@@ -1758,23 +1768,20 @@ inline bool make_batch_plan(int m, int n, int M, int want_S, BatchPlan& bp) {
   const int nblk = n / 128, rbs = m / 128;
   bp.mb = batch_groups(M);
   bp.lds = batch_lds_bytes(M);
-  // Measured on MI355X (K4, 6..128 rows, 4096..28672 output rows): one workgroup per CU is the best fill; every further
-  // split adds partial traffic that grows with the rows (14336x4096, 32 rows: 2 splits 20.3 us, 4 splits 25.8; 128
-  // rows: 43 against 62).  So: the largest split that keeps the grid within the CU count, among the splits that leave
-  // no column range empty.  Splits shorter than 8 column blocks cost more in partial traffic and set-up than their
-  // parallelism returns (4096x4096, 32 rows: 4 splits of 8 blocks 14.8 us, 8 of 4 16.7; 128 rows: 31.7 against 41.4),
-  // unless fewer than half the CUs would have work.
-  const int limit = want_S > 0 ? want_S : (NUM_CU / rbs > 1 ? NUM_CU / rbs : 1);
-  bool found = false, found_long = false;
-  BatchPlan longer = bp;
+  // Measured on MI355X (K4, 6..128 rows, 1024..28672 output rows): one workgroup per CU is the best fill; every further
+  // split adds partial traffic that grows with the rows (14336x4096, 32 rows: 2 splits 19.9 us, 4 splits 24.5; 128
+  // rows: 39 against 48).  So: the largest split that keeps the grid within the CU count, among the splits that leave
+  // no column range empty, and at most 8 of them (the output side requests the slots of up to eight other splits in
+  // one go; 1024x4096 and 2048x4096 at 8..32 rows: 8 splits 11..12 us, 16 splits 11..16, 32 splits 14..22).
+  const int by_cus = NUM_CU / rbs > 1 ? NUM_CU / rbs : 1;
+  const int limit = want_S > 0 ? want_S : (by_cus < 8 ? by_cus : 8);
+  bool found = false;
   for (int S = 1; S <= nblk && S <= limit; ++S) {
     const int cb = (nblk + S - 1) / S;
     if ((nblk + cb - 1) / cb != S) continue;                       // some split would be empty
     if (want_S > 0 && S != want_S) continue;
     bp.S = S; bp.cb = cb; bp.wgs = rbs * S; found = true;
-    if (cb >= 8 && rbs * S >= NUM_CU / 2) { longer = bp; found_long = true; }
   }
-  if (want_S <= 0 && found_long && M > 8) bp = longer;           // with 8 rows the partials are small: keep the fill
   return found;
 }
 

@@ -159,15 +159,17 @@ def test_two_streams_with_their_own_workspaces(dev):
     assert all(torch.equal(o, want_b) for o in outs_b)
 
 
-def test_bounded_wait_gives_up_cleanly(dev, oracle):
-    """The finishing workgroup's wait for the other chunks' partials is bounded.  With the bound forced down to a single
+@pytest.mark.parametrize("M", [1, 32])
+def test_bounded_wait_gives_up_cleanly(dev, oracle, M):
+    """The finishing workgroup's wait for the other chunks' partials is bounded (chunked kernel at 1 row; batched kernel
+    at 32 rows, where the splits of a row block wait for each other).  With the bound forced down to a single
     poll from the host, a launch either comes out right or marks what it could not finish: NaN for those rows and bit 0
     of the workspace's status word; every kernel still runs to its end.  After the bound is restored and the workspace
     cleared, results are right again."""
     from htr_amd import _native, ops
-    print("bounded wait", flush=True)
+    print(f"bounded wait M={M}", flush=True)
     L = _native.lib()
-    qw, sc, su, sv, x = _case(2048, 4096, 4, 1, 4500)
+    qw, sc, su, sv, x = _case(2048, 4096, 4, M, 4500 + M)
     d = [t.to(dev) for t in (qw, sc, su, sv)]
     ref = _ref(oracle, qw, sc, su, sv, x)
     xd = x.to(dev)
@@ -186,7 +188,7 @@ def test_bounded_wait_gives_up_cleanly(dev, oracle):
             yn = y.cpu().numpy()
             bad = ~np.isfinite(yn)
             assert bool(bad.any()) == bool(status & 1)
-            blocks = bad.reshape(1, -1, 128)
+            blocks = bad.reshape(M, -1, 128)
             assert np.all(blocks.all(axis=2) | ~blocks.any(axis=2))         # whole 128-row blocks, never single values
             ok = ~bad
             assert float(np.abs(yn[ok] - ref[ok]).max() / np.abs(ref).max()) <= REL_TOL if ok.any() else True

@@ -39,7 +39,7 @@ def parse():
     ap.add_argument("--viterbi-tiles", type=int, default=0,
                     help="also time the encoder's trellis search on this many 256-weight tiles per K (0 = skip)")
     ap.add_argument("--suite", nargs="*", default=None, metavar="CASE",
-                    help="also time the other baseline configurations (htr_amd/bench_suite.py): table, batch, lm_head, moe, "
+                    help="also time the other baseline configurations (htr_amd/bench_suite.py): table, batch, layer_rows, lm_head, moe, "
                          "prefill; no names = all")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy, so a counter profile of this command holds a kernel of known traffic")

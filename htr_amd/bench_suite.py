@@ -89,6 +89,18 @@ def batch(dev):
     return out
 
 
+def layer_rows(dev):
+    """The four fused linears of the 9B decoder layer (qkv, o, gate_up, down; K4) at 8 .. 128 activation rows: us per
+    launch and their sum per layer, with the tokens/s that sum alone would allow (rows / layer time / 32 layers)."""
+    shapes = (("qkv", 6144, 4096), ("o", 4096, 4096), ("gate_up", 28672, 4096), ("down", 4096, 14336))
+    out = []
+    for M in (8, 16, 32, 64, 128):
+        per = {nm: time_linear(m, n, 4, M, dev)["us"] for nm, m, n in shapes}
+        tot = sum(per.values())
+        out.append({"M": M, "us": per, "us_per_layer": round(tot, 1), "rows_per_s_at_32_layers": round(M / (tot * 32e-6))})
+    return out
+
+
 def lm_head(dev):
     return time_linear(152064, 4096, 4, 1, dev, ring_bytes=1 << 30, launches=24)
 
@@ -190,7 +202,7 @@ def prefill(dev):
     return out
 
 
-CASES = {"table": table, "batch": batch, "lm_head": lm_head, "moe": moe, "prefill": prefill}
+CASES = {"table": table, "batch": batch, "layer_rows": layer_rows, "lm_head": lm_head, "moe": moe, "prefill": prefill}
 
 
 def run(names, dev=None):

@@ -1009,7 +1009,7 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear_batch(const uint32_t* __r
   // row constants of the output side (scale, sign, bias of rows lane and lane + 64), requested ahead of the weight stream by
   // the workgroups that finish rows of the row block, so that they have long arrived when they are needed
   const int RG = (M + 7) >> 3;               // groups of eight activation rows
-  const bool spread = M > 16;                // the splits share the output side (below)
+  const bool spread = M > 16 || (M > 8 && S > 2);   // the splits share the output side (below)
   const bool finisher = spread ? s_idx < RG : s_idx == S - 1;
   const int r0 = rb * 128 + lane, r1 = r0 + 64;
   uint32_t raw_sc0 = 0u, raw_sc1 = 0u, raw_sv0 = 0u, raw_sv1 = 0u, raw_b0 = 0u, raw_b1 = 0u;   // bits only: converted at the end
@@ -1163,8 +1163,8 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear_batch(const uint32_t* __r
   // its partial of those rows in its slot.  So the output side of many rows is spread over the splits instead of
   // falling to one workgroup (32 rows on 4096x14336, 8 splits: 23.0 -> 19.7 us; 128 rows: 56.6 -> 38.5).  The
   // workgroups of one row block are neighbours in dispatch order and the grid fits the chip, so they run together; the
-  // wait is bounded all the same.  Up to 16 rows the last split finishes everything, as in k_linear: two workgroups
-  // that wait for each other cost 0.3 us more than one that waits.
+  // wait is bounded all the same.  Up to 8 rows (one group), and up to 16 rows with two splits, the last split
+  // finishes everything, as in k_linear: two workgroups that wait for each other cost 0.3 us more than one that waits.
   for (int rg = 0, owner = spread ? 0 : S - 1; rg < RG; ++rg, owner = !spread ? owner : (owner + 1 == S ? 0 : owner + 1)) {
     const int mrow = 8 * rg + w;
     if (owner != s_idx && mrow < M) {

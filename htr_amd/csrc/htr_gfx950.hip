@@ -1667,8 +1667,8 @@ inline bool plan_for_chunk(int m, int n, int M, int chunk, Plan& pl) {
 }
 
 // Picks the chunk length (virtual steps per workgroup) with a cost model in microseconds fitted to chunk-length sweeps
-// on MI355X (K4, 1..5 rows, nine shapes from 1024x4096 to 28672x4096, twenty chunk lengths each; the choice is within
-// 0.5 % of the best measured chunk on average, 6 % at worst): a fixed latency chain (launch, x fetch, rotation, partial
+// on MI355X (K4, 1..8 rows, nine shapes from 1024x4096 to 28672x4096, twenty chunk lengths each; the choice is within
+// 1 % of the best measured chunk on average, 10 % at worst): a fixed latency chain (launch, x fetch, rotation, partial
 // exchange, output rotation) that grows with the contributors a finisher reads, eight per round trip; a cost per
 // step that depends on how many workgroups share a CU (one: the workgroup's own decode rate, 0.4 .. 0.5 us; several:
 // throughput bound, proportional to the load of the fullest CU, plus a set-up per workgroup); a penalty for chunks
@@ -1685,7 +1685,7 @@ inline bool make_plan(int m, int n, int M, int nsplit, Plan& pl) {
     return ok;
   }
   if (vtotal >= (long)64 * NUM_CU && nblk <= 64 && plan_for_chunk(m, n, M, nblk, pl)) return true;
-  const double rows = M <= 8 ? 1.0 + 0.08 * (M - 1) : (M <= 16 ? 2.2 : 6.5);
+  const double rows = M <= 8 ? 1.0 + 0.06 * (M - 1) : (M <= 16 ? 2.2 : 6.5);
   double best = 1e30;
   bool found = false;
   const int max_chunk = (int)(vtotal < MAX_CHUNK ? vtotal : MAX_CHUNK);
@@ -1696,16 +1696,16 @@ inline bool make_plan(int m, int n, int M, int nsplit, Plan& pl) {
     const double fill = (double)c.wgs / NUM_CU;
     const bool aligned = (nblk % chunk == 0) || (chunk % nblk == 0);
     const int contributors = chunk >= nblk ? 1 : (nblk + chunk - 1) / chunk;
-    const double steps = chunk * (aligned ? 1.0 : 1.06);
+    const double steps = chunk * (aligned ? 1.0 : 1.06 + 0.04 * (M - 1));
     // one workgroup per CU or fewer: the chip works through `chunk` steps once; more: the fullest CU works through
     // its workgroups one after the other, each with its own set-up and partial hand-over
     // (a grid slightly above one workgroup per CU leaves a few CUs with two: it costs nearly as much as two everywhere)
     const double fill2 = fill < 1.5 ? 1.5 : fill;
-    const double body = fill <= 1.0 ? rows * (0.4 + 0.1 * fill) * steps
-                                    : fill2 * (rows * 0.5 * steps + 0.8 + 0.2 * M);
+    const double body = fill <= 1.0 ? rows * (0.4 + 0.05 * fill) * steps
+                                    : fill2 * (rows * 0.55 * steps + 0.5 + 0.1 * M);
     // hand-over: the contributors' slots are read eight per round trip to memory (0.45 us each)
     const double handover = 0.45 * ((contributors - 1 + 7) / 8);
-    const double t = 4.5 + handover + (c.prerot ? 2.5 : 0.0) + body;
+    const double t = 4.5 + handover + (c.prerot ? 3.0 + 0.1 * M : 0.0) + body;
     if (t < best) { best = t; pl = c; found = true; }
   }
   return found;
@@ -1759,7 +1759,7 @@ template <int K> int launch_linear_k(const LinearLaunch& a, bool prerot, int mb,
 
 // ---- batched kernel: split S of the column blocks per row block
 struct BatchPlan { int S, cb, wgs, mb; size_t lds; };
-constexpr int BATCH_MIN_M = 6;      // rows from which the library policy takes the batched kernel
+constexpr int BATCH_MIN_M = 9;      // rows from which the library policy takes the batched kernel
 inline int batch_groups(int M) { return M <= 16 ? 1 : (M <= 32 ? 2 : (M <= 64 ? 4 : 8)); }   // groups of 16 activation rows
 inline size_t batch_lds_bytes(int M) {
   const int rows = 16 * batch_groups(M);

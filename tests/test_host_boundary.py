@@ -78,6 +78,7 @@ def test_launch_plan_is_consistent(L, m, n, M):
         # activations always rotated ahead
         S = -(-nblk // chunk)
         assert wgs == rbs * S and (S - 1) * chunk < nblk and prerot == 1 and lds <= (64 if M <= 32 else 140) * 1024
+        assert S <= 8 and (wgs <= 256 or S == 1)                                 # the grid fits the chip, at most 8 splits
         # an explicit split is honoured (bit 29 selects the batched kernel)
         assert L.htr_linear_plan(m, n, 4, M, (1 << 29) | 1, out) == 0 and out[0] == nblk and out[1] == rbs
         return

@@ -136,13 +136,15 @@ def test_encode_save_load_plugin_apply(dev, tmp_path):
     assert float((ref - dense).norm() / dense.norm()) < 0.2
 
 
-def test_two_streams_with_their_own_workspaces(dev):
+@pytest.mark.parametrize("Ma,Mb", [(1, 3), (24, 40)])
+def test_two_streams_with_their_own_workspaces(dev, Ma, Mb):
     """Launches of two shapes interleaved on two streams (default priority): the Python layer keeps one workspace per
-    stream, so the partial slots of concurrent launches never meet; every result equals the serial one."""
+    stream, so the partial slots of concurrent launches never meet; every result equals the serial one.  The second
+    case runs the batched kernel on both streams, whose workgroups of one row block wait for each other."""
     from htr_amd import ops
-    print("two streams", flush=True)
-    a = _case(1024, 2048, 4, 1, 4400)
-    b = _case(2048, 1024, 3, 3, 4401)
+    print(f"two streams M={Ma},{Mb}", flush=True)
+    a = _case(1024, 2048, 4, Ma, 4400)
+    b = _case(2048, 1024, 3, Mb, 4401)
     da, xa = [t.to(dev) for t in a[:4]], a[4].to(dev)
     db, xb = [t.to(dev) for t in b[:4]], b[4].to(dev)
     want_a, want_b = ops.linear(xa, *da), ops.linear(xb, *db)

@@ -939,7 +939,7 @@ constexpr int BATCH_FIN_STRIDE = 128 + 4;    // floats per activation row of the
 __device__ __forceinline__ int batch_fin_pos(int r) { return (r & 7) * 16 + (r >> 3); }
 
 template <int K, int MG, int P>
-__global__ __launch_bounds__(WG_THREADS) void k_linear_batch(const uint32_t* __restrict__ qw, float* __restrict__ part,
+__global__ __launch_bounds__(WG_THREADS, MG <= 2 ? 4 : 2) void k_linear_batch(const uint32_t* __restrict__ qw, float* __restrict__ part,
                                                              int m, int n, int M, int S, int flags, const LinearTail t) {
   extern __shared__ __align__(16) unsigned char lds[];
   const int lane = threadIdx.x & 63;
@@ -1759,7 +1759,7 @@ template <int K> int launch_linear_k(const LinearLaunch& a, bool prerot, int mb,
 
 // ---- batched kernel: split S of the column blocks per row block
 struct BatchPlan { int S, cb, wgs, mb; size_t lds; };
-constexpr int BATCH_MIN_M = 9;      // rows from which the library policy takes the batched kernel
+constexpr int BATCH_MIN_M = 9;      // rows from which the library policy takes the batched kernel on every shape
 inline int batch_groups(int M) { return M <= 16 ? 1 : (M <= 32 ? 2 : (M <= 64 ? 4 : 8)); }   // groups of 16 activation rows
 inline size_t batch_lds_bytes(int M) {
   const int rows = 16 * batch_groups(M);
@@ -1810,7 +1810,12 @@ template <int K> int launch_batch_k(const uint32_t* qw, float* part, int m, int 
   }
 }
 // nsplit bit 29: batched kernel with the split in the low bits (0 = policy); otherwise the policy decides by M
-inline bool wants_batch(int M, int nsplit) { return nsplit > 0 ? (nsplit & (1 << 29)) != 0 : M >= BATCH_MIN_M; }
+// Tall matrices (192 row blocks and more) fill the chip without column splits, so the batched kernel needs no exchange
+// there and wins from 6 rows (65536x4096, 8 rows: 41 against 50 us; 152064x4096: 91 against 95).
+inline bool wants_batch(int M, int nsplit, int m) {
+  if (nsplit > 0) return (nsplit & (1 << 29)) != 0;
+  return M >= BATCH_MIN_M || (M >= 6 && m / 128 >= 192);
+}
 
 #define HTR_FOR_K(K, EXPR)                 \
   switch (K) {                             \
@@ -1854,7 +1859,7 @@ float htr_cbscale(void) { return (float)(1.0 / __builtin_sqrt(MEAN_SQ)); }
 
 size_t htr_workspace_bytes(int m, int n, int K, int M, int nsplit) {
   if (K < 2 || K > 8 || !shape_ok(m, n) || M < 1 || M > HTR_MAX_BATCH) return 0;
-  if (wants_batch(M, nsplit)) {
+  if (wants_batch(M, nsplit, m)) {
     BatchPlan bp;
     if (!make_batch_plan(m, n, M, nsplit > 0 ? nsplit & 0xFFFFF : 0, bp)) return 0;
     return ws_need((size_t)bp.wgs * M * 128 * sizeof(float), prerot_bytes(n, M));
@@ -1870,7 +1875,7 @@ int htr_linear_plan(int m, int n, int K, int M, int nsplit, int* out6) {
   if (K < 2 || K > 8) return HTR_ERR_K;
   if (!shape_ok(m, n)) return HTR_ERR_SHAPE;
   if (M < 1 || M > HTR_MAX_BATCH) return HTR_ERR_BATCH;
-  if (wants_batch(M, nsplit)) {
+  if (wants_batch(M, nsplit, m)) {
     BatchPlan bp;
     if (!make_batch_plan(m, n, M, nsplit > 0 ? nsplit & 0xFFFFF : 0, bp)) return HTR_ERR_SPLIT;
     out6[0] = bp.cb; out6[1] = bp.wgs; out6[2] = 1; out6[3] = 1; out6[4] = 1; out6[5] = (int)bp.lds;
@@ -1896,7 +1901,7 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
   if (((uintptr_t)qweight & 15) || ((uintptr_t)scales & 1) || ((uintptr_t)x & (x_dtype == HTR_F32 ? 3 : 1)) ||
       ((uintptr_t)y & (y_dtype == HTR_F32 ? 3 : 1)) || (bias && ((uintptr_t)bias & (y_dtype == HTR_F32 ? 3 : 1))))
     return HTR_ERR_ALIGN;
-  if (wants_batch(M, nsplit)) {
+  if (wants_batch(M, nsplit, m)) {
     BatchPlan bp;
     if (!make_batch_plan(m, n, M, nsplit > 0 ? nsplit & 0xFFFFF : 0, bp)) return HTR_ERR_SPLIT;
     const size_t need = htr_workspace_bytes(m, n, K, M, nsplit);

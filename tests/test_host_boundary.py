@@ -73,7 +73,7 @@ def test_launch_plan_is_consistent(L, m, n, M):
     nblk, rbs = n // 128, m // 128
     need = L.htr_workspace_bytes(m, n, 4, M, 0)
     assert need >= 256 + wgs * M * 128 * 4                                       # header + one partial slot per workgroup
-    if M >= 9:
+    if M >= 9 or (M >= 6 and m // 128 >= 192):
         # batched kernel: `chunk` column blocks per split, S = ceil(nblk / chunk) splits per row block, no empty split,
         # activations always rotated ahead
         S = -(-nblk // chunk)

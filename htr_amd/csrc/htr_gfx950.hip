@@ -29,6 +29,7 @@
 #include <stdint.h>
 #include <string.h>
 #include <stdlib.h>
+#include <atomic>
 #include <type_traits>
 
 #include "../../include/htr_gfx950.h"
@@ -1674,7 +1675,7 @@ inline bool plan_for_chunk(int m, int n, int M, int chunk, Plan& pl) {
 // throughput bound, proportional to the load of the fullest CU, plus a set-up per workgroup); a penalty for chunks
 // that do not tile the rows of column blocks; the extra launch of a pre-rotation; and the growth of all per-step work
 // with the number of activation rows.
-inline bool make_plan(int m, int n, int M, int nsplit, Plan& pl) {
+inline bool search_plan(int m, int n, int M, int nsplit, Plan& pl) {
   const int nblk = n / 128, rbs = m / 128;
   const long vtotal = (long)rbs * nblk;
   pl.mb = M <= 8 ? 1 : (M <= 16 ? 2 : 4);
@@ -1709,6 +1710,37 @@ inline bool make_plan(int m, int n, int M, int nsplit, Plan& pl) {
     if (t < best) { best = t; pl = c; found = true; }
   }
   return found;
+}
+
+// The search above walks every chunk length (up to 4096 of them): tens of microseconds on the host, more than the launch
+// it plans.  Plans depend only on (m, n, M, nsplit), so the last 64 distinct ones are kept.
+inline bool make_plan(int m, int n, int M, int nsplit, Plan& pl) {
+  struct Entry { int m, n, M, nsplit; bool ok; Plan pl; };
+  static Entry cache[64];
+  static int filled = 0, next = 0;
+  static std::atomic_flag busy = ATOMIC_FLAG_INIT;
+  while (busy.test_and_set(std::memory_order_acquire)) {}
+  for (int i = 0; i < filled; ++i) {
+    const Entry& e = cache[i];
+    if (e.m == m && e.n == n && e.M == M && e.nsplit == nsplit) {
+      const bool ok = e.ok;
+      pl = e.pl;
+      busy.clear(std::memory_order_release);
+      return ok;
+    }
+  }
+  busy.clear(std::memory_order_release);
+  Plan found;
+  found.mb = pl.mb;
+  const bool ok = search_plan(m, n, M, nsplit, found);
+  while (busy.test_and_set(std::memory_order_acquire)) {}
+  Entry& e = cache[next];
+  e.m = m; e.n = n; e.M = M; e.nsplit = nsplit; e.ok = ok; e.pl = found;
+  next = (next + 1) % 64;
+  if (filled < 64) ++filled;
+  busy.clear(std::memory_order_release);
+  pl = found;
+  return ok;
 }
 
 // The dispatcher places workgroups wherever resources allow, not evenly: with 512 equal workgroups some CUs receive

@@ -51,17 +51,26 @@ def workspace(device, stream_id, nbytes):
     return _WORKSPACES[keys[0]]
 
 
+_NEED = {}       # workspace bytes per (m, n, K, M, nsplit)
+
+# the current hipStream_t of a device as an integer; the direct accessor skips the construction of a Stream object
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None) or (lambda index: torch.cuda.current_stream(index).cuda_stream)
+
+
 def _launch(x2, qweight, scales, su, sv, bias, y, m, n, K, out_code):
     L = _native.lib()
     M = x2.shape[0]
-    need = L.htr_workspace_bytes(m, n, K, M, NSPLIT)
+    key = (m, n, K, M, NSPLIT)
+    need = _NEED.get(key)
+    if need is None:
+        need = _NEED[key] = L.htr_workspace_bytes(m, n, K, M, NSPLIT)
     if need == 0:
         raise RuntimeError("libhtr_gfx950: no launch plan for this shape / split")
-    stream = torch.cuda.current_stream(x2.device)
-    ws = workspace(x2.device, stream.cuda_stream, need)
+    stream = _raw_stream(x2.device.index)
+    ws = workspace(x2.device, stream, need)
     _native.check(L.htr_linear(qweight.data_ptr(), scales.data_ptr(), su.data_ptr(), sv.data_ptr(), x2.data_ptr(),
                                None if bias is None else bias.data_ptr(), y.data_ptr(), m, n, K, M,
-                               _DTYPE_CODE[x2.dtype], out_code, NSPLIT, ws.data_ptr(), ws.numel(), stream.cuda_stream))
+                               _DTYPE_CODE[x2.dtype], out_code, NSPLIT, ws.data_ptr(), ws.numel(), stream))
 
 
 def _linear_impl(x2, qweight, scales, su, sv, bias, out_dtype=None):
@@ -198,9 +207,16 @@ def _(x2, qweight, scales, su, sv, bias):
 
 
 def linear(x, qweight, scales, su, sv, bias=None):
-    """y = x @ W^T (+bias) for an HTR-W1 weight. x [..., n] -> [..., m] in x.dtype."""
+    """y = x @ W^T (+bias) for an HTR-W1 weight. x [..., n] -> [..., m] in x.dtype.
+
+    Under tracing (torch.compile) the call goes through the registered op `htr::linear`, as in the reference
+    (htr/ops.py:107-122); eager calls skip the dispatcher, which costs more host time than the launch itself."""
     shp = x.shape
-    y = htr_linear_op(x.reshape(-1, shp[-1]), qweight, scales, su, sv, bias)
+    x2 = x.reshape(-1, shp[-1])
+    if torch.compiler.is_compiling():
+        y = htr_linear_op(x2, qweight, scales, su, sv, bias)
+    else:
+        y = _linear_impl(x2.contiguous(), qweight, scales, su, sv, bias)
     return y.reshape(*shp[:-1], qweight.shape[0] * 16)
 
 

@@ -1800,6 +1800,7 @@ inline size_t batch_lds_bytes(int M) {
 }
 inline bool make_batch_plan(int m, int n, int M, int want_S, BatchPlan& bp) {
   const int nblk = n / 128, rbs = m / 128;
+  if ((long)M * n * 2 >= (1L << 31)) return false;          // the kernels address the rotated activations with 32-bit byte offsets
   bp.mb = batch_groups(M);
   bp.lds = batch_lds_bytes(M);
   // Measured on MI355X (K4, 6..128 rows, 1024..28672 output rows): one workgroup per CU is the best fill; every further

@@ -235,30 +235,58 @@ def test_errors(dev):
         ops.linear(x.to(dev), d[0][:, :, :8].contiguous(), d[1], d[2], d[3])      # K = 1
 
 
-@pytest.mark.parametrize("K,m,n", [(4, 4096, 4096), (2, 4096, 4096), (5, 4096, 4096), (4, 14336, 4096),
-                                   (4, 4096, 14336), (3, 14336, 4096)])
-def test_full_size_shapes(dev, oracle, K, m, n):
-    from htr_amd import ops
-    print(f"full size K={K} {m}x{n}", flush=True)
-    qw, sc, su, sv, x = _case(m, n, K, 1, 20261125 + K)
+_WEIGHTS = {}
+
+
+def _weights(m, n, K, seed):
+    """Synthetic HTR-W1 tensors of a full-size case, generated once per (shape, K) and shared by its row counts."""
+    from htr_amd import wire
+    key = (m, n, K, seed)
+    if key not in _WEIGHTS:
+        _WEIGHTS.clear()                                   # one full-size weight at a time in host memory
+        _WEIGHTS[key] = wire.synth_linear(m, n, K, seed)
+    return _WEIGHTS[key]
+
+
+# every cell of the bit-width sweep (K2..K5 x {4096x4096, 14336x4096} x 1, 2, 4 rows), the down projection, and the two
+# fused matrices of the decoder layer as the benchmark launches them (q/k/v and gate/up concatenated along the output dim)
+_FULL = [(K, m, n, M) for K in (2, 3, 4, 5) for (m, n) in ((4096, 4096), (14336, 4096)) for M in (1, 2, 4)]
+_FULL += [(4, 4096, 14336, 1), (4, 6144, 4096, 1), (4, 28672, 4096, 1), (4, 1024, 4096, 1)]
+
+
+@pytest.mark.parametrize("K,m,n,M", _FULL)
+def test_full_size_shapes(dev, oracle, K, m, n, M):
+    from htr_amd import ops, wire
+    print(f"full size K={K} {m}x{n} M={M}", flush=True)
+    qw, sc, su, sv = _weights(m, n, K, 20261125 + K)
+    x = wire.synth_activation(M, n, 20261125 + K + 7 + M)
     d = [t.to(dev) for t in (qw, sc, su, sv)]
     y = ops.linear_f32out(x.to(dev), *d).cpu().numpy()
     ref = _ref(oracle, qw, sc, su, sv, x)
-    assert _rel(y, ref) <= REL_TOL, _rel(y, ref)
+    for r in range(M):
+        assert _rel(y[r], ref[r]) <= REL_TOL, (r, _rel(y[r], ref[r]))
     # linearity in x, a size-independent property: f(2x) == 2 f(x) exactly (power-of-two scaling)
     y2 = ops.linear_f32out((x * 2).to(dev), *d).cpu().numpy()
     assert np.array_equal(y2, 2 * y)
+    # the bf16 output the benchmark times is the round-to-nearest-even cast of the same float32 result
+    yb = ops.linear(x.to(dev), *d)
+    assert yb.dtype == torch.bfloat16
+    assert torch.equal(yb.float().cpu(), torch.from_numpy(y).bfloat16().float())
 
 
-# ---- the small-batch GEMM shapes, the 64-expert stack and the output head as parity cases
-@pytest.mark.parametrize("K,M,m,n", [(3, 8, 14336, 4096), (4, 16, 14336, 4096), (4, 32, 4096, 14336), (3, 32, 14336, 4096),
-                                     (4, 8, 4096, 14336), (4, 64, 14336, 4096), (4, 48, 4096, 14336), (4, 6, 4096, 4096),
-                                     (4, 128, 4096, 4096), (4, 100, 14336, 4096)])
+# ---- the small-batch GEMM shapes (every cell of K3, K4 x 8, 16, 32 rows x gate/up and down), larger row counts, the
+# 64-expert stack and the output head as parity cases
+_BATCH = [(K, M, m, n) for K in (3, 4) for (m, n) in ((14336, 4096), (4096, 14336)) for M in (8, 16, 32)]
+_BATCH += [(4, 64, 14336, 4096), (4, 48, 4096, 14336), (4, 6, 4096, 4096), (4, 128, 4096, 4096), (4, 100, 14336, 4096)]
+
+
+@pytest.mark.parametrize("K,M,m,n", _BATCH)
 def test_small_batch_gemm_shapes(dev, oracle, K, M, m, n, monkeypatch):
-    from htr_amd import ops
+    from htr_amd import ops, wire
     print(f"small-batch K={K} M={M} {m}x{n}", flush=True)
     monkeypatch.setattr(ops, "GEMV_LOOP_MAX", 1 << 30)     # the fused kernel at every M
-    qw, sc, su, sv, x = _case(m, n, K, M, 4000 + 13 * K + M)
+    qw, sc, su, sv = _weights(m, n, K, 4000 + 13 * K)
+    x = wire.synth_activation(M, n, 4000 + 13 * K + M)
     y = ops.linear_f32out(x.to(dev), *[t.to(dev) for t in (qw, sc, su, sv)]).cpu().numpy()
     ref = _ref(oracle, qw, sc, su, sv, x)
     for r in range(M):

@@ -3,14 +3,14 @@ names (K x shape x batch table, 8..128 activation rows, routed experts, lm_head)
 
 Every case cycles through a ring of distinct weight copies larger than the caches (>= 1 GB, or as many copies as
 fit), replays the ring as one HIP graph and reads HIP events on the launch stream.  Used by `bench.py --suite`;
-`python -m htr_amd.bench_suite [names]` prints the same dictionary as JSON.
+`python bench_suite.py [names]` prints the same dictionary as JSON.
 """
 import json
 import sys
 
 import torch
 
-from . import _native, ops, wire
+from htr_amd import _native, ops, wire
 
 HBM_PEAK_GBS = 8000.0
 SEED = 20261125

@@ -31,6 +31,8 @@ SIGNATURES = {
     "htr_grouped_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "htr_linear_grouped": (_i, [_vp, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
     "htr_set_spin_limit": (None, [_i]),
+    "htr_workspace_init": (_i, [_vp, _sz, _vp, _vp]),
+    "htr_stream_capture_id": (ctypes.c_ulonglong, [_vp]),
     "htr_viterbi_workspace_bytes": (_sz, [_i64, _i, _i]),
     "htr_viterbi": (_i, [_vp, _vp, _i64, _i, _i, _i, _vp, _vp, _sz, _vp]),
     "htr_decode_raw": (_i, [_vp, _vp, _i64, _i, _vp]),

@@ -452,6 +452,20 @@ template <int K, typename F> __device__ __forceinline__ void decode_step_mid(con
 // that the number of loads in flight behind any buffer is the same on every path and the wait in front of a decode
 // leaves the other P - 1 loads outstanding.
 #define HTR_PIN() __builtin_amdgcn_sched_barrier(0)
+
+// A finisher that gave up waiting: bit 0 of the workspace's status word (word 0 of the header), and, if the caller
+// registered one (bytes 8..15 of the header: the address of a host-visible word), a flag in host memory, so that the
+// host can see the failure without a device-to-host copy.  Rare path, one lane.
+__device__ __forceinline__ void report_give_up(uint32_t* status) {
+  __hip_atomic_fetch_or(status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const unsigned long long mirror = __hip_atomic_load((const unsigned long long*)(status + 2), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (mirror != 0ull) __hip_atomic_store((uint32_t*)mirror, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+// A workspace whose status word is set holds partials that nobody collected: every later launch on it marks all its
+// outputs NaN (instead of adding stale partials to good ones) until the caller has cleared it (htr_workspace_init).
+__device__ __forceinline__ uint32_t load_status(const uint32_t* status) {
+  return __hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 constexpr int FLAG_LANES = 1 << 4;     // kernel flag: chunk ids are dealt to the XCDs in eight lanes (see k_linear)
 
 template <int K, int MB, int P, int D, bool PREROT>
@@ -849,6 +863,7 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
   if constexpr (PREROT) {
     if (w < nfin * M) row_load(rb_first + (M == 1 ? w : w / M), first_raw);
   }
+  const uint32_t stale = load_status(t.status);     // non-zero: an earlier launch on this workspace gave up
   __syncthreads();
   for (int idx = w; idx < nfin * M; idx += WG_WAVES) {
     const int seg = M == 1 ? idx : idx / M, mrow = idx - seg * M, rb = rb_first + seg;
@@ -899,9 +914,10 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
           __hip_atomic_store(pp + lane + 64, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
       } else if (lane == 0) {
-        __hip_atomic_fetch_or(t.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        report_give_up(t.status);
       }
     }
+    failed |= stale != 0u;
     const float* own = s_fin + ((size_t)seg * M + mrow) * 128;
     v0s += own[lane]; v1s += own[lane + 64];
     // the row scale applies before the output rotation; the sign and 1/sqrt(128) after it
@@ -1177,6 +1193,7 @@ __global__ __launch_bounds__(WG_THREADS, MG <= 2 ? 4 : 2) void k_linear_batch(co
     }
   }
   if (!finisher) return;
+  const uint32_t stale = load_status(t.status);     // non-zero: an earlier launch on this workspace gave up
 
   // ---- output side of this split's row groups: add the other splits' partials (fixed order), finish
   const float rs0 = f16_bits_to_float((uint16_t)raw_sc0) * t.cbscale * INV_SQRT128;
@@ -1224,9 +1241,10 @@ __global__ __launch_bounds__(WG_THREADS, MG <= 2 ? 4 : 2) void k_linear_batch(co
           __hip_atomic_store(pp + lane + 64, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
       } else if (lane == 0) {
-        __hip_atomic_fetch_or(t.status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        report_give_up(t.status);
       }
     }
+    failed |= stale != 0u;
     const float* own = s_fin + mrow * BATCH_FIN_STRIDE;
     const float* oth = own + M * BATCH_FIN_STRIDE;
     v0s += own[pos0] + oth[pos0]; v1s += own[pos1] + oth[pos1];
@@ -1621,6 +1639,15 @@ __global__ __launch_bounds__(VitCfg<K>::THREADS) void k_viterbi(const float* __r
   }
 }
 
+// ------------------------------------------------------------------------------------------------ workspace set-up
+// Zeroes the first `bytes` (a multiple of 16) of a workspace and writes the header's mirror address.  A kernel, not a
+// memset, so that it can be recorded into a HIP graph.
+__global__ __launch_bounds__(256) void k_workspace_init(u4* __restrict__ ws, size_t bytes, unsigned long long mirror) {
+  const size_t n16 = bytes / 16;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n16; i += (size_t)gridDim.x * 256)
+    ws[i] = i == 0 ? u4{0u, 0u, (uint32_t)mirror, (uint32_t)(mirror >> 32)} : u4{0u, 0u, 0u, 0u};
+}
+
 // ------------------------------------------------------------------------------------------------ host side
 thread_local int g_last_hip_error = 0;
 int g_spin_limit = 1 << 20;     // polls (about a microsecond each) before a finishing workgroup gives up
@@ -1730,8 +1757,7 @@ inline bool make_plan(int m, int n, int M, int nsplit, Plan& pl) {
     }
   }
   busy.clear(std::memory_order_release);
-  Plan found;
-  found.mb = pl.mb;
+  Plan found = {};
   const bool ok = search_plan(m, n, M, nsplit, found);
   while (busy.test_and_set(std::memory_order_acquire)) {}
   Entry& e = cache[next];
@@ -1754,6 +1780,31 @@ inline size_t balanced_lds_request(size_t needed, int grid) {
   return share > needed ? share : needed;
 }
 
+// One launch with the runtime's own return value (hipGetLastError after a launch macro would also report an earlier,
+// unrelated failure of the thread as this launch's).
+template <typename T> struct same_type { typedef T type; };
+template <typename... KArgs>
+hipError_t launch_kernel(void (*kern)(KArgs...), dim3 grid, dim3 block, size_t lds, hipStream_t st, typename same_type<KArgs>::type... args) {
+  void* argv[] = {(void*)&args...};
+  return hipLaunchKernel((const void*)kern, grid, block, argv, lds, st);
+}
+// Kernels that may ask for more than the default 48 KB of dynamic LDS get the limit raised to the whole 160 KB once per
+// (kernel, device), not per launch with the launch's own value: the attribute is state of the function, and two host
+// threads that set different values around their launches would race.
+constexpr int MAX_DYNAMIC_LDS = 160 * 1024;
+template <auto Kern> hipError_t allow_full_lds() {
+  static std::atomic<uint64_t> done{0};
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  const uint64_t bit = (uint64_t)1 << (dev & 63);
+  if (done.load(std::memory_order_acquire) & bit) return hipSuccess;
+  e = hipFuncSetAttribute((const void*)Kern, hipFuncAttributeMaxDynamicSharedMemorySize, MAX_DYNAMIC_LDS);
+  if (e == hipSuccess) done.fetch_or(bit, std::memory_order_release);
+  return e;
+}
+#define HTR_CHECK_HIP(EXPR) do { hipError_t e_ = (EXPR); if (e_ != hipSuccess) { g_last_hip_error = (int)e_; return HTR_ERR_LAUNCH; } } while (0)
+
 struct LinearLaunch {
   const uint32_t* qw; const void* x; const uint8_t* su; float* part;
   int m, n, M, chunk, flags, problems;
@@ -1764,15 +1815,10 @@ struct LinearLaunch {
 template <int K, int MB, bool DEEP, bool PREROT> int launch_linear_v(const LinearLaunch& a, int grid, size_t lds, hipStream_t st) {
   constexpr int P = K <= 4 ? 4 : (K <= 6 ? 3 : 2);          // wave-steps of weights in flight
   constexpr int D = DEEP && P >= 4 ? 4 : 2;                 // steps decoded ahead of the activation exchange
-  auto kern = k_linear<K, MB, P, D, PREROT>;
   lds = balanced_lds_request(lds, grid * a.problems);
-  if (lds > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
-  }
-  hipLaunchKernelGGL(kern, dim3(grid, a.problems), dim3(WG_THREADS), lds, st, a.qw, a.x, a.su, a.part, a.m, a.n, a.M, a.chunk, a.flags, a.nblk_magic, a.tail);
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
+  HTR_CHECK_HIP((allow_full_lds<k_linear<K, MB, P, D, PREROT>>()));
+  HTR_CHECK_HIP(launch_kernel(k_linear<K, MB, P, D, PREROT>, dim3(grid, a.problems), dim3(WG_THREADS), lds, st, a.qw, a.x, a.su, a.part,
+                              a.m, a.n, a.M, a.chunk, a.flags, a.nblk_magic, a.tail));
   return HTR_OK;
 }
 // Short chunks are decoded completely ahead of the activation exchange (more registers, so only for one activation
@@ -1822,15 +1868,9 @@ inline bool make_batch_plan(int m, int n, int M, int want_S, BatchPlan& bp) {
 
 template <int K, int MB> int launch_batch_v(const uint32_t* qw, float* part, int m, int n, int M, int flags, const LinearTail& t,
                                             const BatchPlan& bp, hipStream_t st) {
-  auto kern = k_linear_batch<K, MB, 4>;
-  size_t lds = balanced_lds_request(bp.lds, bp.wgs);
-  if (lds > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
-  }
-  hipLaunchKernelGGL(kern, dim3(bp.S, m / 128), dim3(WG_THREADS), lds, st, qw, part, m, n, M, bp.S, flags, t);
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
+  const size_t lds = balanced_lds_request(bp.lds, bp.wgs);
+  HTR_CHECK_HIP((allow_full_lds<k_linear_batch<K, MB, 4>>()));
+  HTR_CHECK_HIP(launch_kernel(k_linear_batch<K, MB, 4>, dim3(bp.S, m / 128), dim3(WG_THREADS), lds, st, qw, part, m, n, M, bp.S, flags, t));
   return HTR_OK;
 }
 template <int K> int launch_batch_k(const uint32_t* qw, float* part, int m, int n, int M, int flags, const LinearTail& t,
@@ -1875,7 +1915,7 @@ const char* htr_strerror(int status) {
     case HTR_ERR_NULL: return "a required pointer is NULL";
     case HTR_ERR_K: return "unsupported K (HTR-W1 allows 2..8)";
     case HTR_ERR_SHAPE: return "m and n must be positive multiples of 128";
-    case HTR_ERR_BATCH: return "M must be in 1..32 for one launch";
+    case HTR_ERR_BATCH: return "M must be in 1..128 for one launch (1..32 for a grouped problem or an explicit chunked plan)";
     case HTR_ERR_DTYPE: return "dtype must be bf16 (0), f16 (1) or f32 (2)";
     case HTR_ERR_WORKSPACE: return "workspace too small or not 256-byte aligned";
     case HTR_ERR_ALIGN: return "tensor pointer not aligned (qweight 16 B, others natural)";
@@ -1923,6 +1963,24 @@ int htr_linear_plan(int m, int n, int K, int M, int nsplit, int* out6) {
 
 void htr_set_spin_limit(int polls) { g_spin_limit = polls < 1 ? 1 : polls; }
 
+int htr_workspace_init(void* workspace, size_t workspace_bytes, void* host_status_word, void* stream) {
+  if (!workspace) return HTR_ERR_NULL;
+  if (workspace_bytes < 2 * WS_HEADER || ((uintptr_t)workspace & 255) || ((uintptr_t)host_status_word & 3)) return HTR_ERR_WORKSPACE;
+  const size_t half = ws_half(workspace_bytes);
+  const size_t n16 = half / 16;
+  const unsigned blocks = (unsigned)(n16 / 256 < 1 ? 1 : (n16 / 256 > 2048 ? 2048 : n16 / 256));
+  HTR_CHECK_HIP(launch_kernel(k_workspace_init, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (u4*)workspace, half,
+                              (unsigned long long)(uintptr_t)host_status_word));
+  return HTR_OK;
+}
+
+unsigned long long htr_stream_capture_id(void* stream) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  unsigned long long id = 0;
+  if (hipStreamGetCaptureInfo((hipStream_t)stream, &status, &id) != hipSuccess) { (void)hipGetLastError(); return 0; }
+  return status == hipStreamCaptureStatusActive ? (id != 0 ? id : ~0ull) : 0;
+}
+
 int htr_linear(const void* qweight, const void* scales, const void* su, const void* sv, const void* x, const void* bias,
                void* y, int m, int n, int K, int M, int x_dtype, int y_dtype, int nsplit, void* workspace,
                size_t workspace_bytes, void* stream) {
@@ -1951,10 +2009,8 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
     t.chunk_magic = 0;
     t.group = nullptr; t.group_prerot_stride = 0; t.group_part_stride = 0;
     hipStream_t st = (hipStream_t)stream;
-    hipLaunchKernelGGL(k_rotate, dim3((n / 128 + WG_WAVES - 1) / WG_WAVES, M), dim3(WG_THREADS), 0, st, x, (const uint8_t*)su, n, x_dtype,
-                       (_Float16*)t.xt_g, (float*)t.xs_g, (float*)t.sc_g, (const htr_group_entry*)nullptr, 0ull);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
+    HTR_CHECK_HIP(launch_kernel(k_rotate, dim3((n / 128 + WG_WAVES - 1) / WG_WAVES, M), dim3(WG_THREADS), 0, st, x, (const uint8_t*)su, n, x_dtype,
+                                (_Float16*)t.xt_g, (float*)t.xs_g, (float*)t.sc_g, (const htr_group_entry*)nullptr, 0ull));
     float* part = (float*)((unsigned char*)workspace + WS_HEADER);
     const int flags = x_dtype | (y_dtype << 2);
     HTR_FOR_K(K, return launch_batch_k<KK>((const uint32_t*)qweight, part, m, n, M, flags, t, bp, st));
@@ -1997,10 +2053,8 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
     t.xt_g = (const _Float16*)wsp;
     t.xs_g = (const float*)(wsp + align256((size_t)M * n * 2));
     t.sc_g = (const float*)(wsp + align256((size_t)M * n * 2) + align256((size_t)M * (n / 128) * 16));
-    hipLaunchKernelGGL(k_rotate, dim3((n / 128 + WG_WAVES - 1) / WG_WAVES, M), dim3(WG_THREADS), 0, st, x, (const uint8_t*)su, n, x_dtype, (_Float16*)t.xt_g,
-                       (float*)t.xs_g, (float*)t.sc_g, (const htr_group_entry*)nullptr, 0ull);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
+    HTR_CHECK_HIP(launch_kernel(k_rotate, dim3((n / 128 + WG_WAVES - 1) / WG_WAVES, M), dim3(WG_THREADS), 0, st, x, (const uint8_t*)su, n, x_dtype,
+                                (_Float16*)t.xt_g, (float*)t.xs_g, (float*)t.sc_g, (const htr_group_entry*)nullptr, 0ull));
   }
   HTR_FOR_K(K, return launch_linear_k<KK>(a, prerot, pl.mb, pl.wgs, pl.lds, st));
   return HTR_OK;
@@ -2069,11 +2123,9 @@ int htr_linear_grouped(const htr_group_entry* entries, int count, int m, int n, 
   t.chunk_magic = (((unsigned long long)1 << 40) + (unsigned)pl.chunk - 1) / (unsigned)pl.chunk;
   t.group = entries; t.group_prerot_stride = pre; t.group_part_stride = (unsigned long long)pl.wgs * max_M * 128;
   hipStream_t st = (hipStream_t)stream;
-  hipLaunchKernelGGL(k_rotate, dim3((n / 128 + WG_WAVES - 1) / WG_WAVES, max_M, count), dim3(WG_THREADS), 0, st, (const void*)nullptr,
-                     (const uint8_t*)nullptr, n, x_dtype, (_Float16*)t.xt_g, (float*)t.xs_g, (float*)t.sc_g, entries,
-                     (unsigned long long)pre);
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
+  HTR_CHECK_HIP(launch_kernel(k_rotate, dim3((n / 128 + WG_WAVES - 1) / WG_WAVES, max_M, count), dim3(WG_THREADS), 0, st, (const void*)nullptr,
+                              (const uint8_t*)nullptr, n, x_dtype, (_Float16*)t.xt_g, (float*)t.xs_g, (float*)t.sc_g, entries,
+                              (unsigned long long)pre));
   HTR_FOR_K(K, return launch_linear_k<KK>(a, true, pl.mb, pl.wgs, pl.lds, st));
   return HTR_OK;
 }
@@ -2095,12 +2147,10 @@ int htr_viterbi(const void* x, const void* w, int64_t tiles, int T, int K, int t
   const double rms = __builtin_sqrt(MEAN_SQ);
 #define HTR_LAUNCH_VIT(KK_)                                                                                              \
   {                                                                                                                      \
-    auto kern = k_viterbi<KK_>;                                                                                          \
     const size_t lds = ((size_t)2 * VitCfg<KK_>::SJ + 2048 + 1024 + 512 + 64) * sizeof(float);                           \
-    hipError_t e0 = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);       \
-    if (e0 != hipSuccess) { g_last_hip_error = (int)e0; return HTR_ERR_LAUNCH; }                                         \
-    hipLaunchKernelGGL(kern, dim3((unsigned)tiles), dim3(VitCfg<KK_>::THREADS), lds, st, (const float*)x, (const float*)w, T,  \
-                       tailbite ? 1 : 0, (uint8_t*)workspace, (uint16_t*)states_u16, rms);                               \
+    HTR_CHECK_HIP((allow_full_lds<k_viterbi<KK_>>()));                                                                   \
+    HTR_CHECK_HIP(launch_kernel(k_viterbi<KK_>, dim3((unsigned)tiles), dim3(VitCfg<KK_>::THREADS), lds, st, (const float*)x, \
+                                (const float*)w, T, tailbite ? 1 : 0, (uint8_t*)workspace, (uint16_t*)states_u16, rms)); \
   }
   switch (K) {
     case 2: HTR_LAUNCH_VIT(2); break;
@@ -2111,8 +2161,6 @@ int htr_viterbi(const void* x, const void* w, int64_t tiles, int T, int K, int t
     default: HTR_LAUNCH_VIT(7); break;
   }
 #undef HTR_LAUNCH_VIT
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
   return HTR_OK;
 }
 
@@ -2123,10 +2171,8 @@ int htr_decode_raw(const void* qweight, void* out_i16, int64_t ntiles, int K, vo
   if (((uintptr_t)qweight & 15) || ((uintptr_t)out_i16 & 15)) return HTR_ERR_ALIGN;
   const int64_t blocks = (ntiles * 8 + 255) / 256;
   hipStream_t st = (hipStream_t)stream;
-  HTR_FOR_K(K, hipLaunchKernelGGL(k_decode_raw<KK>, dim3((unsigned)blocks), dim3(256), 0, st, (const uint32_t*)qweight,
-                                  (int16_t*)out_i16, ntiles));
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
+  HTR_FOR_K(K, HTR_CHECK_HIP(launch_kernel(k_decode_raw<KK>, dim3((unsigned)blocks), dim3(256), 0, st, (const uint32_t*)qweight,
+                                           (int16_t*)out_i16, ntiles)));
   return HTR_OK;
 }
 
@@ -2142,16 +2188,12 @@ int htr_dequant_w(const void* qweight, const void* scales, const void* su, const
   const float cb = htr_cbscale();
 #define HTR_LAUNCH_DQW(KK_)                                                                                              \
   {                                                                                                                      \
-    auto kern = k_dequant_w<KK_>;                                                                                        \
-    hipError_t e0 = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);       \
-    if (e0 != hipSuccess) { g_last_hip_error = (int)e0; return HTR_ERR_LAUNCH; }                                         \
-    hipLaunchKernelGGL(kern, grid, dim3(512), lds, st, (const uint32_t*)qweight, (const uint16_t*)scales,                \
-                       (const uint8_t*)su, (const uint8_t*)sv, (uint16_t*)out_bf16, n / 16, cb);                         \
+    HTR_CHECK_HIP((allow_full_lds<k_dequant_w<KK_>>()));                                                                 \
+    HTR_CHECK_HIP(launch_kernel(k_dequant_w<KK_>, grid, dim3(512), lds, st, (const uint32_t*)qweight, (const uint16_t*)scales, \
+                                (const uint8_t*)su, (const uint8_t*)sv, (uint16_t*)out_bf16, n / 16, cb));               \
   }
   HTR_FOR_K(K, HTR_LAUNCH_DQW(KK));
 #undef HTR_LAUNCH_DQW
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
   return HTR_OK;
 }
 
@@ -2163,10 +2205,8 @@ int htr_dequant_q(const void* qweight, const void* scales, void* out_f32, int mt
   const int64_t blocks = ((int64_t)mt * nt * 8 + 255) / 256;
   hipStream_t st = (hipStream_t)stream;
   const double rms = __builtin_sqrt(MEAN_SQ);
-  HTR_FOR_K(K, hipLaunchKernelGGL(k_dequant_q<KK>, dim3((unsigned)blocks), dim3(256), 0, st, (const uint32_t*)qweight,
-                                  (const uint16_t*)scales, (float*)out_f32, mt, nt, rms));
-  hipError_t e = hipGetLastError();
-  if (e != hipSuccess) { g_last_hip_error = (int)e; return HTR_ERR_LAUNCH; }
+  HTR_FOR_K(K, HTR_CHECK_HIP(launch_kernel(k_dequant_q<KK>, dim3((unsigned)blocks), dim3(256), 0, st, (const uint32_t*)qweight,
+                                           (const uint16_t*)scales, (float*)out_f32, mt, nt, rms)));
   return HTR_OK;
 }
 

@@ -27,28 +27,80 @@ NSPLIT = int(os.environ.get("HTR_NSPLIT", "0"))
 # dequantize + GEMM 42 / 73 / 105 us; two fused launches (256 rows) no longer beat it.
 GEMV_LOOP_MAX = int(os.environ.get("HTR_GEMV_LOOP_MAX", "128"))
 
-_WORKSPACES = {}
+class _Workspace:
+    """One device buffer for split partials and pre-rotated activations, with its failure flag in pinned host memory."""
+    __slots__ = ("buf", "flag", "stream")
+
+    def __init__(self, buf, flag, stream):
+        self.buf, self.flag, self.stream = buf, flag, stream
+
+
+_WORKSPACES = {}      # (device index, stream) or (device index, "capture", capture id) -> _Workspace
+_RETIRED = []         # buffers that a capture in progress has already recorded launches with: never freed
+_FLAG_POOLS = {}      # device index -> [pinned int32 tensor, its numpy view, next free word]
+_FLAG_WORDS = 1024
+
+
+def _flag_word(device):
+    """A 4-byte word of pinned host memory (None while a capture is in progress and no pool exists yet, or when the
+    pool is used up: the workspace then works without a host-side flag)."""
+    pool = _FLAG_POOLS.get(device.index)
+    if pool is None:
+        if torch.cuda.is_current_stream_capturing():
+            return None
+        t = torch.zeros(_FLAG_WORDS, dtype=torch.int32).pin_memory()
+        pool = _FLAG_POOLS[device.index] = [t, t.numpy(), 0]
+    if pool[2] >= _FLAG_WORDS:
+        return None
+    i = pool[2]
+    pool[2] += 1
+    return pool[1][i:i + 1], pool[0].data_ptr() + 4 * i
+
+
+def _heal(ws, device):
+    """A launch on this workspace gave up waiting (its host flag is set): drain the device, clear the workspace, raise."""
+    torch.cuda.synchronize(device)
+    ws.flag[0][0] = 0
+    _native.check(_native.lib().htr_workspace_init(ws.buf.data_ptr(), ws.buf.numel(), ws.flag[1], ws.stream))
+    torch.cuda.synchronize(device)
+    raise RuntimeError("libhtr_gfx950: an earlier launch on this workspace gave up waiting for a partial result "
+                       "(its outputs, and those of every launch after it, are NaN); the workspace has been cleared")
+
+
+def check_status(device=None):
+    """Raises if any launch so far gave up waiting on one of the workspaces of `device` (all devices if None), after
+    clearing that workspace.  Eager calls check their own workspace by themselves; this is for graph replays."""
+    for key, ws in list(_WORKSPACES.items()):
+        if (device is None or key[0] == torch.device(device).index) and ws.flag is not None and ws.flag[0][0] != 0:
+            _heal(ws, torch.device("cuda", key[0]))
 
 
 def workspace(device, stream_id, nbytes):
-    """Zeroed scratch for split partials and pre-rotated activations, one per (device, stream).
+    """Scratch for split partials and pre-rotated activations: one per (device, stream), and one per HIP-graph capture.
 
     The reference keeps one counter tensor per device (htr/ops.py:24-28), which two streams
     would corrupt; keying by stream keeps concurrent streams apart.  Kernels leave the
-    partial slots zero, so the buffer is zeroed only when it is (re)allocated.
-    Calls recorded into a HIP graph use one more buffer per device, shared by every capture (a capture runs on a
-    stream of its own, and replays of one device's graphs are not expected to overlap).  Every eager call makes sure
-    that buffer exists and is large enough for its own shape, so that a capture that follows a warm-up pass over the
-    same shapes allocates nothing and records no fill.
+    partial slots zero, so a buffer is cleared only when it is created (by the library's fill kernel).
+    Every capture gets buffers of its own (keyed by the runtime's capture id), allocated inside the capture, i.e. from
+    the graph's memory pool, and kept alive here for good: its address is part of the recorded launches.  A buffer
+    that a capture has used is never replaced or freed; if a later call of the same capture needs more, a further
+    buffer is added.  Eager calls never touch a capture's buffers.
     """
-    capturing = torch.cuda.is_current_stream_capturing()
-    keys = [(device.index, "capture")] if capturing else [(device.index, stream_id), (device.index, "capture")]
-    for key in keys:
-        ws = _WORKSPACES.get(key)
-        if ws is None or ws.numel() < nbytes:
-            size = max(int(nbytes), 1 << 20)
-            _WORKSPACES[key] = torch.zeros(size, dtype=torch.uint8, device=device)
-    return _WORKSPACES[keys[0]]
+    cid = _native.lib().htr_stream_capture_id(stream_id) if torch.cuda.is_current_stream_capturing() else 0
+    key = (device.index, "capture", cid) if cid else (device.index, stream_id)
+    ws = _WORKSPACES.get(key)
+    if ws is not None and ws.buf.numel() >= nbytes:
+        if ws.flag is not None and ws.flag[0][0] != 0 and not cid:
+            _heal(ws, device)
+        return ws.buf
+    if ws is not None and cid:
+        _RETIRED.append(ws)
+    size = max(int(nbytes), 1 << 20)
+    buf = torch.empty(size, dtype=torch.uint8, device=device)
+    flag = _flag_word(device)
+    ws = _WORKSPACES[key] = _Workspace(buf, flag, stream_id)
+    _native.check(_native.lib().htr_workspace_init(buf.data_ptr(), size, None if flag is None else flag[1], stream_id))
+    return buf
 
 
 _NEED = {}       # workspace bytes per (m, n, K, M, nsplit)
@@ -210,11 +262,12 @@ def linear(x, qweight, scales, su, sv, bias=None):
     """y = x @ W^T (+bias) for an HTR-W1 weight. x [..., n] -> [..., m] in x.dtype.
 
     Under tracing (torch.compile) the call goes through the registered op `htr::linear`, as in the reference
-    (htr/ops.py:107-122); eager calls skip the dispatcher, which costs more host time than the launch itself."""
+    (htr/ops.py:107-122), and so do tensor subclasses (fake and functional tensors of other tracers); eager calls on
+    plain tensors skip the dispatcher, which costs more host time than the launch itself."""
     shp = x.shape
     x2 = x.reshape(-1, shp[-1])
-    if torch.compiler.is_compiling():
-        y = htr_linear_op(x2, qweight, scales, su, sv, bias)
+    if torch.compiler.is_compiling() or type(x2) is not torch.Tensor or type(qweight) not in (torch.Tensor, torch.nn.Parameter):
+        y = htr_linear_op(x2, qweight, scales, su, sv, bias)      # tracing, fake or functional tensors: the registered op
     else:
         y = _linear_impl(x2.contiguous(), qweight, scales, su, sv, bias)
     return y.reshape(*shp[:-1], qweight.shape[0] * 16)

@@ -62,7 +62,9 @@ float htr_cbscale(void);
  * allocates it once, zeroes it once, and may reuse it for any later call whose requirement
  * is not larger, as long as calls that share a workspace are ordered on one stream: kernels
  * leave the partial slots zero on exit.  The first 32-bit word stays zero unless a kernel
- * gave up waiting for a partial (see htr_set_spin_limit).
+ * gave up waiting for a partial (see htr_set_spin_limit and htr_workspace_init for what follows).
+ * Thread safety: calls from several host threads are safe as long as launches that share a
+ * workspace are ordered on one stream.
  * The library splits the buffer at workspace_bytes / 2: the first half holds the status word and the
  * partial slots (the part that must be zero), the second half is scratch.  Pass the same
  * workspace_bytes whenever you pass the same buffer, so that the split stays where it was;
@@ -72,6 +74,28 @@ float htr_cbscale(void);
  * nsplit: as in htr_linear.
  */
 size_t htr_workspace_bytes(int m, int n, int K, int M, int nsplit);
+
+/*
+ * Prepares (or clears) a workspace on `stream` with a fill kernel (no memset, so the call may be recorded into a HIP
+ * graph): zeroes the half that must be zero, status word included, and stores `host_status_word` in bytes 8..15 of the
+ * 256-byte header.  host_status_word is NULL or the address of a 4-byte word in pinned, device-visible host memory
+ * (hipHostMalloc) that the caller has set to 0: a kernel that gives up waiting also stores 1 there, so the host can
+ * notice the failure by reading its own memory, without a copy or a synchronisation.
+ * Failure protocol: a launch that gives up marks its unfinished rows NaN and sets bit 0 of the status word (word 0 of
+ * the workspace); the partials it did not collect stay in the slots.  From then on every launch on that workspace marks
+ * ALL its outputs NaN, until the caller, after the stream has drained, calls htr_workspace_init again.
+ * A caller that zeroes a fresh workspace itself (memset) and never registers a host word needs no call to this.
+ * Reference: the zeroed per-device counter tensor of htr/ops.py:24-28 (which has no failure path: its kernels wait
+ * without bound).
+ */
+int htr_workspace_init(void* workspace, size_t workspace_bytes, void* host_status_word, void* stream);
+
+/*
+ * 0 if `stream` is not being captured into a HIP graph, otherwise a non-zero id that is unique to the capture in
+ * progress (hipStreamGetCaptureInfo).  Lets a host layer give every capture a workspace of its own, which must then
+ * live as long as the graph.  Reference: none (torch.cuda.is_current_stream_capturing is the nearest).
+ */
+unsigned long long htr_stream_capture_id(void* stream);
 
 /*
  * The launch plan htr_linear would use: out6 = {steps (128x128 weight blocks of one row block, walked row-major)

@@ -41,6 +41,12 @@ def test_constants(L, oracle):
     from htr_amd import wire
     assert wire.cbscale() == oracle.c_cbscale()
     assert L.htr_strerror(0) == b"ok" and b"K" in L.htr_strerror(2)
+    # the batch message names the limits the header declares
+    from htr_amd import _native
+    msg = L.htr_strerror(4).decode()
+    assert f"1..{_native.MAX_BATCH}" in msg and f"1..{_native.MAX_GROUP_ROWS}" in msg
+    assert L.htr_workspace_init(None, 1 << 20, None, None) == 1          # NULL workspace: refused before any GPU call
+    assert L.htr_workspace_init(256, 64, None, None) == 6                # too small
 
 
 def test_validation_codes_without_gpu(L):

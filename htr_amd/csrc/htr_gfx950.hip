@@ -44,7 +44,10 @@ constexpr float SQRT128 = 11.313708498984761f;
 constexpr double MEAN_SQ = 1433042863.0 / 65536.0;
 
 typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+typedef __bf16 b8 __attribute__((ext_vector_type(8)));
 typedef float f4 __attribute__((ext_vector_type(4)));
+typedef float f2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u2 __attribute__((ext_vector_type(2)));
 
@@ -293,9 +296,9 @@ struct LinearTail {
   unsigned long long group_part_stride;     // floats
 };
 
-constexpr int ROT_PAIRS = 16;  // (activation row, 128-column block) pairs a workgroup may rotate by itself
+constexpr int ROT_PAIRS = 32;  // (activation row, 128-column block) pairs a workgroup may rotate by itself: four per wave
 
-// LDS layout (dynamic): [xt: (M + 1) rows x row_halves f16][xs: M * nbl * 2 f32 (per tile parity)][sc: M f32][pmax: 16 f32]
+// LDS layout (dynamic): [xt: (M + 1) rows x row_halves f16][xs: M * nbl * 2 f32 (per tile parity)][sc: M f32][bs: 32 f32, scale per pair]
 //                       [fin: segfin x M x 128 f32, partials of the row blocks this workgroup finishes]
 // nbl = number of distinct column blocks a chunk touches = min(chunk, n / 128)
 // One rotated 128-column block is stored as [columns 0..7 of tiles 0..7][columns 8..15 of tiles 0..7] (2 x 64 halves), and
@@ -318,6 +321,16 @@ __device__ __forceinline__ int scale_exponent(float amax) {
   return max(-100, ex - 127 - 13);
 }
 __device__ __forceinline__ float pow2f(int e) { return __uint_as_float((uint32_t)(127 + e) << 23); }
+// Scale exponent of one rotated 128-column block from the bit pattern of its largest |value| (after the 1/sqrt(128)):
+// 0 while that lies in [2^-8, 2^15) -- no f16 overflow, and values down to 2^-6 of the largest stay normal -- else the
+// exponent that brings it to [2^13, 2^14).  Zero, denormal, infinite and NaN maxima keep scale 1.
+__device__ __forceinline__ int block_scale_exponent(uint32_t amax_bits) {
+  const int ex = (int)((amax_bits >> 23) & 0xFFu);
+  if (ex == 0 || ex == 255) return 0;
+  const int l2 = ex - 127;
+  if (l2 >= -8 && l2 <= 14) return 0;
+  return max(-100, l2 - 13);
+}
 
 // Rotation of all activation rows ahead of the linear kernel (used where every workgroup rotating its own column
 // blocks would repeat too much work, and for float32 activations).  Workgroup (g, row) rotates column blocks
@@ -467,6 +480,7 @@ __device__ __forceinline__ uint32_t load_status(const uint32_t* status) {
   return __hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 constexpr int FLAG_LANES = 1 << 4;     // kernel flag: chunk ids are dealt to the XCDs in eight lanes (see k_linear)
+constexpr int FLAG_LANE_LEN_SHIFT = 8; // with FLAG_LANES: grid / 8 in the bits from here up (no read of the hidden grid-size argument)
 
 template <int K, int MB, int P, int D, bool PREROT>
 __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restrict__ qw_a, const void* __restrict__ x_a,
@@ -480,17 +494,19 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
   float* __restrict__ part = part_a;
   int M = M_a;
   LinearTail t = t_a;
-  if (t_a.group != nullptr) {              // uniform: one entry of the problem table per blockIdx.y
-    const htr_group_entry& ge = t_a.group[blockIdx.y];
-    M = ge.M;
-    if (M <= 0) return;
-    qw = (const uint32_t*)ge.qweight; x = ge.x; su = (const uint8_t*)ge.su;
-    part = part_a + (size_t)blockIdx.y * t_a.group_part_stride;
-    t.scales = (const uint16_t*)ge.scales; t.sv = (const uint8_t*)ge.sv; t.bias = ge.bias; t.y = ge.y;
-    const size_t shift = (size_t)blockIdx.y * t_a.group_prerot_stride;
-    t.xt_g = (const _Float16*)((const unsigned char*)t_a.xt_g + shift);
-    t.xs_g = (const float*)((const unsigned char*)t_a.xs_g + shift);
-    t.sc_g = (const float*)((const unsigned char*)t_a.sc_g + shift);
+  if constexpr (PREROT) {                    // grouped launches always come with pre-rotated activations
+    if (t_a.group != nullptr) {              // uniform: one entry of the problem table per blockIdx.y
+      const htr_group_entry& ge = t_a.group[blockIdx.y];
+      M = ge.M;
+      if (M <= 0) return;
+      qw = (const uint32_t*)ge.qweight; x = ge.x; su = (const uint8_t*)ge.su;
+      part = part_a + (size_t)blockIdx.y * t_a.group_part_stride;
+      t.scales = (const uint16_t*)ge.scales; t.sv = (const uint8_t*)ge.sv; t.bias = ge.bias; t.y = ge.y;
+      const size_t shift = (size_t)blockIdx.y * t_a.group_prerot_stride;
+      t.xt_g = (const _Float16*)((const unsigned char*)t_a.xt_g + shift);
+      t.xs_g = (const float*)((const unsigned char*)t_a.xs_g + shift);
+      t.sc_g = (const float*)((const unsigned char*)t_a.sc_g + shift);
+    }
   }
   const int lane = threadIdx.x & 63;
   const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));   // wave index, provably uniform: keeps the
@@ -502,7 +518,7 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
   // one row block run on one XCD and the partial hand-over between them stays on that XCD's side of the memory
   // system.  A finisher still waits only for chunks of its own row block, i.e. for workgroups b - 8, b - 16, ...
   int cid = (int)blockIdx.x;
-  if (flags & FLAG_LANES) cid = ((int)blockIdx.x & 7) * ((int)gridDim.x >> 3) + ((int)blockIdx.x >> 3);
+  if (flags & FLAG_LANES) cid = ((int)blockIdx.x & 7) * (flags >> FLAG_LANE_LEN_SHIFT) + ((int)blockIdx.x >> 3);
   const int v0 = cid * chunk, nsteps = min(vtotal, v0 + chunk) - v0;
   // v / nblk for v < 2^24 by multiplication: nblk_magic = ceil(2^40 / nblk)
   auto div_nblk = [&](int v) { return (int)(((unsigned long long)(unsigned)v * nblk_magic) >> 40); };
@@ -518,23 +534,24 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
   _Float16* xt = (_Float16*)lds;
   float* s_xs = (float*)(lds + (size_t)(M + 1) * rowh * 2);
   float* s_sc = s_xs + 2 * M * nblmax;                 // activation scale per row
-  float* s_pmax = s_sc + M;                            // max|x| per (row, block) pair
+  float* s_bs = s_sc + M;                              // power-of-two scale per (row, block) pair this workgroup rotated
   float* s_fin = (float*)(lds + lds_fin_offset(M, nblmax));
 
   const int npairs = M * nbl;
   // pair index -> activation row: pi / nbl for pi < 2^16 through the float reciprocal (the quotient's fraction is at
   // least 0.5 / nbl away from an integer, far more than the rounding error), instead of an integer division per use
-  const float inv_nbl = 1.0f / (float)nbl;
+  const float inv_nbl = __builtin_amdgcn_rcpf((float)nbl);
   auto row_of_pair = [&](int pi) { return M == 1 ? 0 : (int)(((float)pi + 0.5f) * inv_nbl); };
   auto pair_col = [&](int li) { int b = all_blocks ? li : c0 + li; if (b >= nblk) b -= nblk; return b * 128; };
 
-  // ---- activations first: they head the longest dependency chain.  Wave w rotates the (row, block) pairs w and w + 8:
-  // one dword (two 16-bit elements) per lane and pair, plus the su byte that holds the two sign bits.  Descriptors
-  // over x and su: a pair beyond the chunk's last one gets an out-of-range offset and reads zeros, so the loads
-  // issue back to back without branches.
-  constexpr int NPW = ROT_PAIRS / WG_WAVES;   // pairs per wave
-  uint32_t xr[NPW], sb[NPW];
-  int prow[NPW], pli[NPW];
+  // ---- activations first: they head the longest dependency chain.  Wave w rotates the (row, block) pairs 4w .. 4w + 3
+  // on the matrix unit: H128 = H4 (x) H32 over the element index i = 32 a + c, so a block is a 4 x 32 matrix X and
+  // H128 x = H4 . X . H32.  The four pairs of a wave are the 16 rows (pair p, a) of one MFMA A operand: lane
+  // (k-group gk = lane / 16, row = lane % 16 = 4 p + a) loads the 8 consecutive elements 32 a + 8 gk .. + 7 of its pair
+  // (16 bytes) and the one su byte that holds their signs.  Descriptors over x and su: a pair beyond the chunk's last
+  // one gets an out-of-range offset and reads zeros, so the loads issue back to back without branches.
+  u4 xr = {0u, 0u, 0u, 0u};
+  uint32_t sb = 0u;
   constexpr int COPY_REGS = 4;
   u4 cp[COPY_REGS];
   int cdst[COPY_REGS];
@@ -545,23 +562,15 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
     constexpr int OUT_OF_RANGE = 0x7FFFFF00;
     // every offset first, then the loads back to back: with address arithmetic (and its branches) between two loads
     // the compiler waits for the first load to return before it issues the second one and the weight stream behind it
-    int xoff[NPW], soff[NPW];
-#pragma unroll
-    for (int tt = 0; tt < NPW; ++tt) {
-      const int pi = w + tt * WG_WAVES;
-      const bool live = pi < npairs;
-      prow[tt] = row_of_pair(pi);
-      pli[tt] = pi - prow[tt] * nbl;
-      const int col = pair_col(pli[tt]);
-      xoff[tt] = live ? (prow[tt] * n + col) * 2 + 4 * lane : OUT_OF_RANGE;
-      soff[tt] = live ? (col >> 3) + (lane >> 2) : OUT_OF_RANGE;
-    }
+    const int pi = 4 * w + ((lane & 15) >> 2), a = lane & 3, gk = lane >> 4;
+    const bool live = pi < npairs;
+    const int prow = row_of_pair(pi), pli = pi - prow * nbl;
+    const int col = pair_col(pli) + 32 * a + 8 * gk;
+    const int xoff = live ? (prow * n + col) * 2 : OUT_OF_RANGE;
+    const int soff = live ? col >> 3 : OUT_OF_RANGE;
     HTR_PIN();
-#pragma unroll
-    for (int tt = 0; tt < NPW; ++tt) {
-      xr[tt] = __builtin_amdgcn_raw_buffer_load_b32(xrsrc, xoff[tt], 0, 0);
-      sb[tt] = (uint32_t)(uint8_t)__builtin_amdgcn_raw_buffer_load_b8(srsrc, soff[tt], 0, 0);
-    }
+    xr = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xoff, 0, 0);
+    sb = (uint32_t)(uint8_t)__builtin_amdgcn_raw_buffer_load_b8(srsrc, soff, 0, 0);
     HTR_PIN();
   } else {
     // with pre-rotated activations: 16-byte pieces of this chunk's x~ slice, through a descriptor over x~ so that the
@@ -615,9 +624,8 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
     b0v = cvt(r.b0); b1v = cvt(r.b1);
   };
   RowRaw first_raw = {0u, 0u, 0u, 0u, 0u, 0u};
-  if constexpr (!PREROT) {
-    if (w < nfin * M) row_load(rb_first + (M == 1 ? w : w / M), first_raw);
-  }
+  const bool early_rows = !PREROT && M == 1;       // more rows: requested before the last barrier (no division up here)
+  if (early_rows && w < nfin) row_load(rb_first + w, first_raw);
 
   // ---- the weight stream.  This wave's strip of row block rb is tile row rb * 8 + w; its 8 tiles of column block blk
   // are 64 * K contiguous dwords; a strip is contiguous over blk, the same strip of the next row block starts 8 strips
@@ -644,65 +652,100 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
 
   for (int i = threadIdx.x; i < rowh / 2; i += WG_THREADS) ((uint32_t*)(xt + (size_t)M * rowh))[i] = 0u;   // zero row
 
-  // ---- rotation, first half: unpack, apply su, publish max|x| of the pair, rotate unscaled in float32 (H128 is
-  // linear and the scale is a power of two, so scaling afterwards gives the same bits)
-  float ra[NPW], rb[NPW];
+  // ---- rotation (waves that have a pair): signs, X . H32 as two matrix instructions (exact: the operands are the
+  // 16-bit activations themselves and +-1, accumulated in float32), H4 over the four accumulator registers, then the
+  // block's own power-of-two scale, rounding to f16 and the sums per tile parity.  A block keeps scale 1 unless its
+  // largest rotated value would leave f16's comfortable range (then 2^e brings it to [2^13, 2^14)): ordinary
+  // activations have scale 1 in every block and the product accumulates across blocks inside the matrix unit; if any
+  // block of the chunk has another scale, the products are scaled per block (see consume()).  No exchange between
+  // waves, so one barrier between the rotation and the first product.
   if constexpr (!PREROT) {
-    const bool is_bf16 = x_dtype == HTR_BF16;
+    if (4 * w < npairs) {                                            // uniform
+      const bool is_bf16 = x_dtype == HTR_BF16;
+      uint32_t xs4[4] = {xr.x, xr.y, xr.z, xr.w};
 #pragma unroll
-    for (int tt = 0; tt < NPW; ++tt) {
-      const int pi = w + tt * WG_WAVES;
-      uint32_t lo, hi;
-      if (is_bf16) { lo = xr[tt] << 16; hi = xr[tt] & 0xFFFF0000u; }
-      else { lo = __float_as_uint(f16_bits_to_float((uint16_t)xr[tt])); hi = __float_as_uint(f16_bits_to_float((uint16_t)(xr[tt] >> 16))); }
-      const int sh = 2 * (lane & 3);                                 // bits of elements 2 lane, 2 lane + 1 in the su byte
-      lo ^= ((sb[tt] >> sh) & 1u) << 31;
-      hi ^= ((sb[tt] >> (sh + 1)) & 1u) << 31;
-      ra[tt] = __uint_as_float(lo); rb[tt] = __uint_as_float(hi);
-      if (pi < npairs) {                                             // uniform
-        const float mx = wave_max(fmaxf(fabsf(ra[tt]), fabsf(rb[tt])));
-        if (lane == 0) s_pmax[pi] = mx;
-        // lane holds elements 2 lane and 2 lane + 1: the in-lane stage is index bit 0, lane bit i is index bit i + 1
-        fwht128_wave(ra[tt], rb[tt], lane);
+      for (int d = 0; d < 4; ++d)                                    // elements 2d (low half), 2d + 1 (high half): su bits 2d, 2d + 1
+        xs4[d] ^= ((sb << (15 - 2 * d)) & 0x8000u) | ((sb << (30 - 2 * d)) & 0x80000000u);
+      // B operand: H32[k][c'] = (-1)^popcount(k & c') for k = 8 gk + i (dword d holds i = 2d, 2d + 1) and
+      // c' = 16 h + j, j = lane % 16; as 16-bit ones with the sign bit set where the parity is odd
+      const int j = lane & 15, gk = lane >> 4;
+      const uint32_t one2 = is_bf16 ? 0x3F803F80u : 0x3C003C00u;
+      const uint32_t o1 = (j & 1) ? 0x80000000u : 0u;
+      const uint32_t e1 = (j & 2) ? 0x80008000u : 0u;
+      const uint32_t e2 = (j & 4) ? 0x80008000u : 0u;
+      const uint32_t f3 = ((gk & 1) && (j & 8)) ? 0x80008000u : 0u;   // k bit 3 with c' bit 3
+      const uint32_t f4m = (gk & 2) ? 0x80008000u : 0u;               // k bit 4 with c' bit 4 (h = 1)
+      const uint32_t b0 = one2 ^ o1 ^ f3;
+      const u4 hb0 = {b0, b0 ^ e1, b0 ^ e2, b0 ^ e1 ^ e2};
+      const u4 hb1 = {hb0.x ^ f4m, hb0.y ^ f4m, hb0.z ^ f4m, hb0.w ^ f4m};
+      const u4 xa = {xs4[0], xs4[1], xs4[2], xs4[3]};
+      const f4 zero4 = {0.f, 0.f, 0.f, 0.f};
+      f4 t0, t1;
+      if (is_bf16) {
+        t0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(b8, xa), __builtin_bit_cast(b8, hb0), zero4, 0, 0, 0);
+        t1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(b8, xa), __builtin_bit_cast(b8, hb1), zero4, 0, 0, 0);
+      } else {
+        t0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, xa), __builtin_bit_cast(h8, hb0), zero4, 0, 0, 0);
+        t1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, xa), __builtin_bit_cast(h8, hb1), zero4, 0, 0, 0);
+      }
+      // D: lane (p = lane / 16, j), register a: T[p][a][16 h + j].  H4 over a gives element 32 a' + 16 h + j.
+      float y[2][4];
+      {
+        const float u0 = t0.x + t0.y, u1 = t0.x - t0.y, u2 = t0.z + t0.w, u3 = t0.z - t0.w;
+        y[0][0] = u0 + u2; y[0][1] = u1 + u3; y[0][2] = u0 - u2; y[0][3] = u1 - u3;
+        const float w0 = t1.x + t1.y, w1 = t1.x - t1.y, w2 = t1.z + t1.w, w3 = t1.z - t1.w;
+        y[1][0] = w0 + w2; y[1][1] = w1 + w3; y[1][2] = w0 - w2; y[1][3] = w1 - w3;
+      }
+      // largest |value| of the pair: 8 in the lane, then over the 16 lanes of the row
+      float mx = fmaxf(fmaxf(fmaxf(fabsf(y[0][0]), fabsf(y[0][1])), fmaxf(fabsf(y[0][2]), fabsf(y[0][3]))),
+                       fmaxf(fmaxf(fabsf(y[1][0]), fabsf(y[1][1])), fmaxf(fabsf(y[1][2]), fabsf(y[1][3]))));
+      uint32_t mu = __float_as_uint(mx * INV_SQRT128);               // non-negative floats compare like their bit patterns
+      mu = max(mu, dpp_mov_u32<0xB1>(mu)); mu = max(mu, dpp_mov_u32<0x4E>(mu));
+      mu = max(mu, dpp_mov_u32<0x141>(mu)); mu = max(mu, dpp_mov_u32<0x140>(mu));
+      const int e = block_scale_exponent(mu);
+      const float f = pow2f(-e) * INV_SQRT128;
+      const int po = 4 * w + (lane >> 4);
+      const bool live_o = po < npairs;
+      const int prow_o = row_of_pair(po), pli_o = po - prow_o * nbl;
+      _Float16* dst = xt + (size_t)prow_o * rowh + pli_o * 128 + (j >> 3) * 64 + (j & 7);
+      float sums[2];
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const h2 p01 = __builtin_convertvector(f2{y[h][0] * f, y[h][1] * f}, h2);
+        const h2 p23 = __builtin_convertvector(f2{y[h][2] * f, y[h][3] * f}, h2);
+        if (live_o) {                                                // element 32 a' + 16 h + j: tile 2 a' + h, column j
+          dst[(0 + h) * 8] = p01.x; dst[(2 + h) * 8] = p01.y; dst[(4 + h) * 8] = p23.x; dst[(6 + h) * 8] = p23.y;
+        }
+        // sum of the rounded values of tile parity h: in the lane, then over the row
+        float sh = __builtin_amdgcn_fdot2(p23, h2{(_Float16)1.f, (_Float16)1.f}, __builtin_amdgcn_fdot2(p01, h2{(_Float16)1.f, (_Float16)1.f}, 0.f, false), false);
+        sh += dpp_mov<0xB1>(sh); sh += dpp_mov<0x4E>(sh); sh += dpp_mov<0x141>(sh); sh += dpp_mov<0x140>(sh);
+        sums[h] = sh;
+      }
+      if (live_o && j == 0) {
+        s_xs[2 * po] = sums[0]; s_xs[2 * po + 1] = sums[1];
+        s_bs[po] = pow2f(e);
       }
     }
   }
 
-  // ---- decode the first D steps into registers around the activation exchange: they need no x~, and they fill the
-  // time the other waves take to reach the barriers (short chunks are decoded completely this way)
+  // ---- decode the first D steps into registers ahead of the barrier: they need no x~, and they fill the time the
+  // rotating waves take (short chunks are decoded completely this way)
   static_assert(D >= 2 && D <= P && D % 2 == 0, "pre-decoded steps come out of the first D stream buffers");
   const int hist = history_lane_byteaddr(lane);
   DecodedStep<K> pre[D];
 #pragma unroll
-  for (int i = 0; i < D / 2; ++i) {
+  for (int i = 0; i < D; ++i) {
     if (i == 0 || i < nsteps) decode_step<K>(buf[i], hist, pre[i]);
     prefetch(buf[i]);
   }
-
-  if constexpr (!PREROT) {
-    __syncthreads();
-    // rotation, second half: the row's scale from the published maxima, then scale, round to f16, store
+  // The decoded operands are first used behind the barrier, in conditional code, and the compiler would sink the
+  // whole decode down there (after the barrier, where nothing overlaps it any more): pin the values here.
 #pragma unroll
-    for (int tt = 0; tt < NPW; ++tt) {
-      const int pi = w + tt * WG_WAVES;
-      if (pi < npairs) {
-        const float amax = wave_max(s_pmax[prow[tt] * nbl + min(lane, nbl - 1)]);
-        const int e = scale_exponent(amax);
-        const float f = pow2f(-e) * INV_SQRT128;
-        if (pli[tt] == 0 && lane == 0) s_sc[prow[tt]] = pow2f(e);
-        const _Float16 ha = (_Float16)(ra[tt] * f), hb = (_Float16)(rb[tt] * f);
-        const uint32_t packed = (uint32_t)__builtin_bit_cast(uint16_t, ha) | ((uint32_t)__builtin_bit_cast(uint16_t, hb) << 16);
-        *(uint32_t*)(xt + (size_t)prow[tt] * rowh + pli[tt] * 128 + xt_slot(2 * lane)) = packed;
-        // sum of the rounded x~ per tile parity: element 2 lane sits in tile lane / 8, so the parity is lane bit 3
-        float s = (float)ha + (float)hb;
-        s += lane_xor_dpp<1>(s); s += lane_xor_dpp<2>(s); s += lane_xor_dpp<4>(s);
-        float e0, o0;
-        halves16(s, e0, o0); s = e0 + o0;
-        halves32(s, e0, o0); s = e0 + o0;
-        if ((lane & ~8) == 0) s_xs[2 * pi + (lane >> 3)] = s;
-      }
-    }
-  } else {
+  for (int i = 0; i < D; ++i)
+#pragma unroll
+    for (int k = 0; k < 4; ++k) asm volatile("" : "+v"(pre[i].a[k]));
+
+  if constexpr (PREROT) {
     // copy the slice into LDS; sums per (row, block, parity) come with it
 #pragma unroll
     for (int tt = 0; tt < COPY_REGS; ++tt) {
@@ -718,11 +761,6 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
       const int pi = i >> 1, mrow = row_of_pair(pi), li = pi - mrow * nbl;
       s_xs[i] = t.xs_g[((size_t)mrow * nblk + (pair_col(li) >> 7)) * 4 + (i & 1)];
     }
-  }
-#pragma unroll
-  for (int i = D / 2; i < D; ++i) {
-    if (i < nsteps) decode_step<K>(buf[i], hist, pre[i]);
-    prefetch(buf[i]);
   }
   __syncthreads();
 
@@ -748,9 +786,13 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
     offs[mb] = 0.f; sc[mb] = 0.f;
     if (live) {
       if constexpr (PREROT) sc[mb] = t.sc_g[mrow];
-      else sc[mb] = s_sc[mrow];
+      else sc[mb] = 1.f;
     }
   }
+  // does any block this workgroup rotated carry a scale other than 1?  (uniform; never with pre-rotated activations,
+  // whose scale is one per row)
+  bool scaled = false;
+  if constexpr (!PREROT) scaled = __any(s_bs[min(lane, npairs - 1)] != 1.f) != 0;
 
   f4 acc[MB][2];
 #pragma unroll
@@ -761,9 +803,10 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
   // previous step's matrix instructions issue, so that their latency hides behind the decode
   h8 B0[MB], B1[MB];
   float xsv[MB];
+  float bsv[MB];     // the block's scale (only read where some block's scale is not 1)
   float k1534[MB];
 #pragma unroll
-  for (int mb = 0; mb < MB; ++mb) k1534[mb] = xsoff[mb] >= 0 ? 1534.f : 0.f;
+  for (int mb = 0; mb < MB; ++mb) { k1534[mb] = xsoff[mb] >= 0 ? 1534.f : 0.f; bsv[mb] = 1.f; }
   auto load_b = [&](int li) {
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
@@ -772,20 +815,42 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
       B1[mb] = *(const h8*)(bp + 64);
       xsv[mb] = s_xs[max(xsoff[mb], 0) + 2 * li];
     }
+    if constexpr (!PREROT) {
+      if (scaled) {
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) bsv[mb] = s_bs[(max(xsoff[mb], 0) >> 1) + li];
+      }
+    }
   };
   load_b(cur_li);
   // product of the decoded step with the chunk's rotated activations, and the end of a segment
   auto consume = [&](const DecodedStep<K>& d, bool maybe_last) {
+    if (PREROT || !scaled) {
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) acc[mb][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[0], B0[mb], acc[mb][0], 0, 0, 0);
+      for (int mb = 0; mb < MB; ++mb) acc[mb][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[0], B0[mb], acc[mb][0], 0, 0, 0);
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) acc[mb][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[2], B0[mb], acc[mb][1], 0, 0, 0);
+      for (int mb = 0; mb < MB; ++mb) acc[mb][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[2], B0[mb], acc[mb][1], 0, 0, 0);
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) acc[mb][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[1], B1[mb], acc[mb][0], 0, 0, 0);
+      for (int mb = 0; mb < MB; ++mb) acc[mb][0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[1], B1[mb], acc[mb][0], 0, 0, 0);
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) acc[mb][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[3], B1[mb], acc[mb][1], 0, 0, 0);
+      for (int mb = 0; mb < MB; ++mb) acc[mb][1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[3], B1[mb], acc[mb][1], 0, 0, 0);
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) offs[mb] = __builtin_fmaf(k1534[mb], xsv[mb], offs[mb]);
+      for (int mb = 0; mb < MB; ++mb) offs[mb] = __builtin_fmaf(k1534[mb], xsv[mb], offs[mb]);
+    } else {
+      // blocks with different scales: the block's product on its own, then into the running sums in true units
+      const f4 zero4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+#pragma unroll
+        for (int rr = 0; rr < 2; ++rr) {
+          f4 pr = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[2 * rr], B0[mb], zero4, 0, 0, 0);
+          pr = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[2 * rr + 1], B1[mb], pr, 0, 0, 0);
+#pragma unroll
+          for (int jj = 0; jj < 4; ++jj) acc[mb][rr][jj] = __builtin_fmaf(pr[jj], bsv[mb], acc[mb][rr][jj]);
+        }
+        offs[mb] = __builtin_fmaf(k1534[mb] * xsv[mb], bsv[mb], offs[mb]);
+      }
+    }
     ++done; ++cur_blk; ++cur_li;
     const bool row_end = cur_blk == nblk;
     const bool last = maybe_last && done == nsteps;
@@ -860,9 +925,7 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
   // pairs w, w + 8, ...
   const size_t slot_floats = (size_t)M * 128;
   if (nfin == 0) return;        // a pure contributor: its partial is on its way, nothing else to do (uniform)
-  if constexpr (PREROT) {
-    if (w < nfin * M) row_load(rb_first + (M == 1 ? w : w / M), first_raw);
-  }
+  if (!early_rows && w < nfin * M) row_load(rb_first + (M == 1 ? w : w / M), first_raw);
   const uint32_t stale = load_status(t.status);     // non-zero: an earlier launch on this workspace gave up
   __syncthreads();
   for (int idx = w; idx < nfin * M; idx += WG_WAVES) {
@@ -2037,7 +2100,7 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
   {
     static const bool lanes_on = getenv("HTR_LANES") == nullptr || atoi(getenv("HTR_LANES")) != 0;
     const int nblk = n / 128, rbs = m / 128;
-    if (lanes_on && pl.chunk < nblk && nblk % pl.chunk == 0 && rbs % 8 == 0 && rbs >= 16 && pl.wgs % 8 == 0) a.flags |= FLAG_LANES;
+    if (lanes_on && pl.chunk < nblk && nblk % pl.chunk == 0 && rbs % 8 == 0 && rbs >= 16 && pl.wgs % 8 == 0) a.flags |= FLAG_LANES | ((pl.wgs / 8) << FLAG_LANE_LEN_SHIFT);
   }
   a.nblk_magic = (((unsigned long long)1 << 40) + (unsigned)(n / 128) - 1) / (unsigned)(n / 128);
   LinearTail& t = a.tail;

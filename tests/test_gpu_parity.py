@@ -265,9 +265,16 @@ def test_full_size_shapes(dev, oracle, K, m, n, M):
     ref = _ref(oracle, qw, sc, su, sv, x)
     for r in range(M):
         assert _rel(y[r], ref[r]) <= REL_TOL, (r, _rel(y[r], ref[r]))
-    # linearity in x, a size-independent property: f(2x) == 2 f(x) exactly (power-of-two scaling)
+    # linearity in x, a size-independent property: f(2x) == 2 f(x).  Power-of-two scaling is exact in every operation of
+    # the path except where a rotated activation falls below 2^-14 and is rounded on f16's denormal grid (a block keeps
+    # scale 1 while its largest rotated value lies in [2^-8, 2^15)): a handful of elements per launch, each off by at
+    # most 2^-25, far below one float32 ulp of an output.  Hence a few-ulp bound instead of bit equality.
     y2 = ops.linear_f32out((x * 2).to(dev), *d).cpu().numpy()
-    assert np.array_equal(y2, 2 * y)
+    assert np.abs(y2 - 2 * y).max() <= 1e-6 * np.abs(y).max()
+    # scaling by 2^20 moves every block to a scale of its own (products are then summed block by block in float32
+    # instead of inside the matrix unit: another rounding order, the same values to float32 accuracy)
+    y3 = ops.linear_f32out((x * float(2 ** 20)).to(dev), *d).cpu().numpy()
+    assert np.abs(y3 - float(2 ** 20) * y).max() <= 1e-5 * float(2 ** 20) * np.abs(y).max()
     # the bf16 output the benchmark times is the round-to-nearest-even cast of the same float32 result
     yb = ops.linear(x.to(dev), *d)
     assert yb.dtype == torch.bfloat16

@@ -268,9 +268,12 @@ def test_full_size_shapes(dev, oracle, K, m, n, M):
     # linearity in x, a size-independent property: f(2x) == 2 f(x).  Power-of-two scaling is exact in every operation of
     # the path except where a rotated activation falls below 2^-14 and is rounded on f16's denormal grid (a block keeps
     # scale 1 while its largest rotated value lies in [2^-8, 2^15)): a handful of elements per launch, each off by at
-    # most 2^-25, far below one float32 ulp of an output.  Hence a few-ulp bound instead of bit equality.
+    # most 2^-25.  The product carries the decode's offset (1534 + v) and the offset's share, 1534 * sum(x~) ~ 1e5, is
+    # taken off in float32 at the end, so such a change can move that difference by one ulp of 1e5: a few 1e-4 in the
+    # first output of a 128-row block, where the output rotation collects what all rows have in common.  Hence a bound
+    # of 1e-5 of max|y| (a hundredth of the parity tolerance) instead of bit equality.
     y2 = ops.linear_f32out((x * 2).to(dev), *d).cpu().numpy()
-    assert np.abs(y2 - 2 * y).max() <= 1e-6 * np.abs(y).max()
+    assert np.abs(y2 - 2 * y).max() <= 1e-5 * np.abs(y).max()
     # scaling by 2^20 moves every block to a scale of its own (products are then summed block by block in float32
     # instead of inside the matrix unit: another rounding order, the same values to float32 accuracy)
     y3 = ops.linear_f32out((x * float(2 ** 20)).to(dev), *d).cpu().numpy()

@@ -15,6 +15,7 @@ BF16, F16, F32 = 0, 1, 2
 MAX_BATCH = 128
 MAX_GROUP_ROWS = 32
 MAX_GROUP = 4096
+STATIC_SCRATCH_BYTES = 8 << 20
 
 _lib = None
 
@@ -28,6 +29,7 @@ SIGNATURES = {
     "htr_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "htr_linear_plan": (_i, [_i, _i, _i, _i, _i, ctypes.POINTER(ctypes.c_int)]),
     "htr_linear": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
+    "htr_linear_static": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "htr_grouped_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "htr_linear_grouped": (_i, [_vp, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
     "htr_set_spin_limit": (None, [_i]),

@@ -2123,6 +2123,42 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
   return HTR_OK;
 }
 
+// ---- htr_linear for callers that can neither allocate nor bring a workspace: the workspace is an array in the
+// library's own device image.  Host code only ever holds the address hipGetSymbolAddress returns for it on the current
+// device (every device has its own copy of the array at its own address; the symbol's name itself is no device address).
+static __device__ __align__(256) unsigned char scratch[HTR_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int MAX_DEVICES = 64;
+void* g_scratch_ptr[MAX_DEVICES];                 // per device: address of `scratch` there, once looked up
+std::atomic<uint64_t> g_scratch_known{0};         // bit d: g_scratch_ptr[d] is valid
+}
+
+int htr_linear_static(const void* qweight, const void* scales, const void* su, const void* sv, const void* x, const void* bias,
+                      void* y, int m, int n, int K, int M, int x_dtype, int y_dtype, int reset, void* stream) {
+  if (K < 2 || K > 8) return HTR_ERR_K;
+  if (!shape_ok(m, n)) return HTR_ERR_SHAPE;
+  if (M < 1 || M > HTR_MAX_BATCH) return HTR_ERR_BATCH;
+  const size_t need = htr_workspace_bytes(m, n, K, M, 0);
+  if (need == 0 || need > (size_t)HTR_STATIC_SCRATCH_BYTES) return HTR_ERR_WORKSPACE;      // beyond the built-in workspace
+  int dev = 0;
+  HTR_CHECK_HIP(hipGetDevice(&dev));
+  if (dev < 0 || dev >= MAX_DEVICES) { g_last_hip_error = (int)hipErrorInvalidDevice; return HTR_ERR_LAUNCH; }
+  const uint64_t bit = (uint64_t)1 << dev;
+  if (!(g_scratch_known.load(std::memory_order_acquire) & bit)) {
+    void* p = nullptr;
+    HTR_CHECK_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    g_scratch_ptr[dev] = p;                       // two threads racing here store the same address
+    g_scratch_known.fetch_or(bit, std::memory_order_release);
+  }
+  void* ws = g_scratch_ptr[dev];
+  if (reset) {
+    const int rc = htr_workspace_init(ws, HTR_STATIC_SCRATCH_BYTES, nullptr, stream);
+    if (rc != HTR_OK) return rc;
+  }
+  return htr_linear(qweight, scales, su, sv, x, bias, y, m, n, K, M, x_dtype, y_dtype, 0, ws, HTR_STATIC_SCRATCH_BYTES, stream);
+}
+
 // plan of a grouped launch: every problem has the same shape, so one plan serves all; the activations are always
 // rotated ahead (one launch for all problems) and the chunk is chosen for the whole grid
 static bool make_group_plan(int count, int m, int n, int max_M, Plan& pl) {

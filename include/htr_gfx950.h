@@ -127,6 +127,27 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
                void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * htr_linear on a workspace that is part of the library: for callers that cannot allocate device memory at the point
+ * of the call and have no workspace to pass (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * allocation).  It has no counterpart in the reference.  The call allocates nothing, frees nothing and calls no
+ * allocating routine; inputs and outputs are the caller's, as in htr_linear, and the launch policy is the library's
+ * (nsplit = 0).  The workspace is an array of HTR_STATIC_SCRATCH_BYTES in the library's device image; every GPU the
+ * library runs on holds its own copy until the process ends.
+ * Limit: problems with htr_workspace_bytes(m, n, K, M, 0) > HTR_STATIC_SCRATCH_BYTES return HTR_ERR_WORKSPACE (all
+ * decode shapes of up to 8 rows fit, 32 rows on 14336 x 4096 too; 64 rows there do not).
+ * All calls on one GPU share that GPU's array: calls that overlap in time on one GPU (different streams or graphs
+ * running concurrently) race on it; order them on one stream.  The array starts zeroed and every launch leaves it as
+ * it must be for the next one; after a launch that gave up waiting (NaN outputs, see htr_workspace_init) pass
+ * reset != 0 once, with the stream drained: the call then clears the array with a fill kernel on `stream` first.
+ * The first call on a device looks the array's address up there (hipGetSymbolAddress); make that call outside of
+ * a graph capture.
+ */
+#define HTR_STATIC_SCRATCH_BYTES (8u << 20)
+int htr_linear_static(const void* qweight, const void* scales, const void* su, const void* sv,
+                      const void* x, const void* bias, void* y,
+                      int m, int n, int K, int M, int x_dtype, int y_dtype, int reset, void* stream);
+
+/*
  * One entry of a grouped launch: the HTR-W1 tensors, activations and output of one problem.  The table lives in
  * DEVICE memory (so that a routing kernel can fill it), is 8-byte aligned and is read by the kernels only.
  */

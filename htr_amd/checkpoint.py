@@ -132,3 +132,137 @@ def save_checkpoint(directory, linears, config=None):
     with open(os.path.join(directory, "config.json"), "w") as f:
         json.dump(cfg, f, indent=2)
     return cfg
+
+
+# ------------------------------------------------------------------------------------------------ routed-expert chunks
+# The reference's routed-expert encoder (htr/moe_encode.py:26-29, 216-225) writes, per layer L and per run of `chunk`
+# consecutive experts starting at e0, one file <root>/L<L>/c<e0:03d>.pt = torch.save of
+#   {"format": "HTR-W1-P2-PACKED-1", "L": L, "K": K,
+#    "experts": [{"e": id, "n": calibration rows, "packed": {role: {"qweight", "scales", "su", "sv"}},
+#                 "what_bf16_sha256": {role: hex}}, ...], "rows": [...], ...}
+# with role in ("gate", "up", "down"), and <root>/PLAN.json with the run's arguments and the same format string.  The
+# sha256 is over the BF16 bits of the encoder's reconstruction, which the encoder checked to equal wire.dequant of the
+# packed tensors bit for bit (htr/moe_encode.py:63-75), so a reader can check a chunk without the encoder.
+PACKED_FORMAT = "HTR-W1-P2-PACKED-1"
+ROLES = ("gate", "up", "down")
+FIELDS = ("qweight", "scales", "su", "sv")
+
+
+def _chunk_name(e0):
+    return f"c{e0:03d}.pt"
+
+
+def write_packed_chunk(path, L, K, experts, extra=None):
+    """Write one chunk file.  experts: iterable of {"e": id, "n": rows, "packed": {role: (qweight, scales, su, sv)}};
+    the reconstruction hashes are computed here from wire.dequant.  For tests and for converters on this side: the
+    reference's own encoder is the normal producer."""
+    import hashlib
+    out = []
+    for ex in experts:
+        packed, sha = {}, {}
+        for role in ROLES:
+            t = tuple(v.detach().cpu().contiguous() for v in ex["packed"][role])
+            if wire.check_shapes(*t)[2] != K:
+                raise ValueError(f"expert {ex['e']} {role}: tensors are not K = {K}")
+            packed[role] = dict(zip(FIELDS, t))
+            sha[role] = hashlib.sha256(wire.dequant(*t).bfloat16().contiguous().view(torch.int16).numpy().tobytes()).hexdigest()
+        out.append({"e": int(ex["e"]), "n": int(ex.get("n", 0)), "packed": packed, "what_bf16_sha256": sha})
+    z = {"format": PACKED_FORMAT, "L": int(L), "K": int(K), "experts": out, "rows": [], **(extra or {})}
+    os.makedirs(os.path.dirname(os.path.abspath(path)), exist_ok=True)
+    torch.save(z, path)
+    return z
+
+
+def read_packed_chunk(path, device="cpu", verify=False):
+    """One chunk file -> {"L", "K", "experts": {e: {"n", "gate", "up", "down", "what_bf16_sha256"}}} with every role an
+    HTR-W1 tuple (qweight, scales, su, sv) on `device`.  The file is unpickled with torch's weights-only loader: tensors,
+    numbers, strings, lists and dicts, nothing that runs code.  verify=True also recomputes the reconstruction hashes
+    (decodes every matrix on the host: slow for real experts)."""
+    z = torch.load(path, map_location="cpu", weights_only=True)
+    if not isinstance(z, dict) or z.get("format") != PACKED_FORMAT:
+        raise ValueError(f"{path}: not a {PACKED_FORMAT} chunk (format = {z.get('format') if isinstance(z, dict) else type(z).__name__!r})")
+    K = int(z["K"])
+    if not 2 <= K <= 8:
+        raise ValueError(f"{path}: K = {K} outside 2..8")
+    experts = {}
+    for ex in z["experts"]:
+        e = int(ex["e"])
+        if e in experts:
+            raise ValueError(f"{path}: expert {e} appears twice")
+        rec = {"n": int(ex.get("n", 0)), "what_bf16_sha256": dict(ex.get("what_bf16_sha256") or {})}
+        for role in ROLES:
+            fields = ex["packed"][role]
+            t = tuple(fields[f] for f in FIELDS)
+            m, n, k = wire.check_shapes(*t)
+            if k != K:
+                raise ValueError(f"{path}: expert {e} {role} has K = {k}, the chunk says {K}")
+            if verify:
+                import hashlib
+                got = hashlib.sha256(wire.dequant(*t).bfloat16().contiguous().view(torch.int16).numpy().tobytes()).hexdigest()
+                want = rec["what_bf16_sha256"].get(role)
+                if want != got:
+                    raise ValueError(f"{path}: expert {e} {role}: decoded matrix does not match the encoder's reconstruction hash")
+            rec[role] = tuple(v.to(device) for v in t)
+        if rec["gate"][0].shape != rec["up"][0].shape or rec["down"][0].shape[0] * 16 != rec["gate"][2].numel() * 8:
+            raise ValueError(f"{path}: expert {e}: gate/up/down shapes do not form an MLP")
+        experts[e] = rec
+    return {"L": int(z["L"]), "K": K, "experts": experts}
+
+
+def fuse_gate_up(gate, up):
+    """gate and up of one expert as the fused [2F, H] HTR-W1 tuple ops.moe_experts takes (gate rows first).  They
+    share the input, so they must share su (the encoder draws one su per group: htr/moe_encode.py:199 shared_su)."""
+    if not torch.equal(gate[2], up[2]):
+        raise ValueError("gate and up do not share the input sign vector: they cannot run as one fused matrix")
+    return (torch.cat([gate[0], up[0]]).contiguous(), torch.cat([gate[1], up[1]]).contiguous(), gate[2],
+            torch.cat([gate[3], up[3]]).contiguous())
+
+
+class PackedExperts:
+    """A directory of routed-expert chunks: <root>/PLAN.json (optional) and <root>/L<L>/c<e0:03d>.pt."""
+
+    def __init__(self, root):
+        self.root = root
+        self.plan = None
+        pf = os.path.join(root, "PLAN.json")
+        if os.path.exists(pf):
+            with open(pf) as f:
+                self.plan = json.load(f)
+            if self.plan.get("format") != PACKED_FORMAT:
+                raise ValueError(f"{pf}: format {self.plan.get('format')!r}, this build reads {PACKED_FORMAT!r}")
+
+    def layers(self):
+        out = []
+        for d in os.listdir(self.root):
+            if d.startswith("L") and d[1:].isdigit() and os.path.isdir(os.path.join(self.root, d)):
+                out.append(int(d[1:]))
+        return sorted(out)
+
+    def chunks(self, L):
+        """Paths of layer L's finished chunks in expert order (claims and temporary files of running encoders are skipped)."""
+        d = os.path.join(self.root, f"L{L}")
+        names = [fn for fn in os.listdir(d) if fn.startswith("c") and fn.endswith(".pt") and fn[1:-3].isdigit()]
+        return [os.path.join(d, fn) for fn in sorted(names, key=lambda fn: int(fn[1:-3]))]
+
+    def layer(self, L, device="cpu", verify=False):
+        """(gate_up, down, K): lists indexed by expert id, ready for ops.moe_experts.  Raises if the layer's chunks leave
+        a hole in the expert ids, disagree in K, or name another layer."""
+        recs, K = {}, None
+        for p in self.chunks(L):
+            z = read_packed_chunk(p, device, verify)
+            if z["L"] != L:
+                raise ValueError(f"{p}: chunk of layer {z['L']} under L{L}")
+            if K is not None and z["K"] != K:
+                raise ValueError(f"{p}: K = {z['K']}, earlier chunks of the layer have {K}")
+            K = z["K"]
+            for e, rec in z["experts"].items():
+                if e in recs:
+                    raise ValueError(f"{p}: expert {e} is in two chunks")
+                recs[e] = rec
+        if not recs:
+            raise FileNotFoundError(f"no chunks for layer {L} under {self.root}")
+        if sorted(recs) != list(range(len(recs))):
+            raise ValueError(f"layer {L}: expert ids {sorted(recs)[:4]}.. are not 0..{len(recs) - 1} (chunks missing?)")
+        gate_up = [fuse_gate_up(recs[e]["gate"], recs[e]["up"]) for e in range(len(recs))]
+        down = [recs[e]["down"] for e in range(len(recs))]
+        return gate_up, down, K

@@ -82,3 +82,79 @@ def test_save_checkpoint_writes_what_the_reader_and_the_plugin_expect(tmp_path):
         assert all(torch.equal(a, b) for a, b in zip(ck.linear(p), want))
     hc = vp.HTRConfig.from_config(qc)
     assert hc.modules == {"layers.0.mlp.gate_proj": 3, "lm_head": 5}
+
+
+# ---- routed-expert chunks (htr/moe_encode.py:26-29, 216-225 of the reference)
+GOLDEN_MOE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "moe_L3")
+
+
+def test_packed_chunk_fixture_reads_and_verifies():
+    pe = checkpoint.PackedExperts(GOLDEN_MOE)
+    assert pe.plan["format"] == "HTR-W1-P2-PACKED-1" and pe.layers() == [3]
+    assert [os.path.basename(p) for p in pe.chunks(3)] == ["c000.pt", "c002.pt"]
+    z = checkpoint.read_packed_chunk(pe.chunks(3)[1], verify=True)
+    assert z["L"] == 3 and z["K"] == 3 and sorted(z["experts"]) == [2, 3] and z["experts"][3]["n"] == 15
+    gate_up, down, K = pe.layer(3, verify=True)
+    assert K == 3 and len(gate_up) == len(down) == 4
+    for e in range(4):
+        assert wire.check_shapes(*gate_up[e]) == (256, 256, 3) and wire.check_shapes(*down[e]) == (256, 128, 3)
+        want = wire.synth_linear(128, 256, 3, 7000 + 10 * e)                 # the seeds tests/golden/make_moe_chunk.py uses
+        assert torch.equal(gate_up[e][0][:8], want[0]) and torch.equal(gate_up[e][1][:128], want[1])
+        assert torch.equal(gate_up[e][2], want[2]) and torch.equal(gate_up[e][3][:16], want[3])
+        assert torch.equal(down[e][0], wire.synth_linear(256, 128, 3, 7002 + 10 * e)[0])
+
+
+def test_packed_chunk_round_trip_and_refusals(tmp_path):
+    def expert(e, K=2, same_su=True):
+        g = wire.synth_linear(128, 128, K, 10 + e)
+        u = wire.synth_linear(128, 128, K, 20 + e)
+        if same_su:
+            u = (u[0], u[1], g[2], u[3])
+        return {"e": e, "n": e, "packed": {"gate": g, "up": u, "down": wire.synth_linear(128, 128, K, 30 + e)}}
+
+    root = tmp_path / "run"
+    checkpoint.write_packed_chunk(str(root / "L0" / "c000.pt"), 0, 2, [expert(0), expert(1)])
+    gate_up, down, K = checkpoint.PackedExperts(str(root)).layer(0, verify=True)
+    assert K == 2 and len(gate_up) == 2 and gate_up[1][0].shape == (16, 8, 16)
+    # a flipped payload bit fails the hash check and only the hash check
+    z = torch.load(str(root / "L0" / "c000.pt"), weights_only=True)
+    z["experts"][0]["packed"]["down"]["qweight"][0, 0, 0] ^= 1
+    torch.save(z, str(root / "L0" / "c000.pt"))
+    checkpoint.read_packed_chunk(str(root / "L0" / "c000.pt"))
+    with pytest.raises(ValueError, match="reconstruction hash"):
+        checkpoint.read_packed_chunk(str(root / "L0" / "c000.pt"), verify=True)
+    # another format string, a hole in the expert ids, gate/up with different su, mixed K in one layer, wrong layer
+    z["format"] = "HTR-W1-P1"
+    torch.save(z, str(tmp_path / "bad.pt"))
+    with pytest.raises(ValueError, match="not a HTR-W1-P2-PACKED-1"):
+        checkpoint.read_packed_chunk(str(tmp_path / "bad.pt"))
+    checkpoint.write_packed_chunk(str(root / "L1" / "c002.pt"), 1, 2, [expert(2), expert(3)])
+    with pytest.raises(ValueError, match="chunks missing"):
+        checkpoint.PackedExperts(str(root)).layer(1)
+    checkpoint.write_packed_chunk(str(root / "L2" / "c000.pt"), 2, 2, [expert(0, same_su=False)])
+    with pytest.raises(ValueError, match="share the input sign"):
+        checkpoint.PackedExperts(str(root)).layer(2)
+    checkpoint.write_packed_chunk(str(root / "L4" / "c000.pt"), 4, 2, [expert(0)])
+    checkpoint.write_packed_chunk(str(root / "L4" / "c001.pt"), 4, 3, [expert(1, K=3)])
+    with pytest.raises(ValueError, match="earlier chunks"):
+        checkpoint.PackedExperts(str(root)).layer(4)
+    checkpoint.write_packed_chunk(str(root / "L5" / "c000.pt"), 6, 2, [expert(0)])
+    with pytest.raises(ValueError, match="under L5"):
+        checkpoint.PackedExperts(str(root)).layer(5)
+    with pytest.raises(ValueError, match="not K = 3"):
+        checkpoint.write_packed_chunk(str(tmp_path / "k.pt"), 0, 3, [expert(0)])
+
+
+def test_packed_chunk_loader_executes_nothing(tmp_path):
+    """A chunk-shaped pickle that carries a callable is refused by the weights-only loader instead of being run."""
+    import pickle
+
+    class Boom:
+        def __reduce__(self):
+            return (os.system, ("true",))
+
+    with open(tmp_path / "evil.pt", "wb") as f:
+        pickle.dump({"format": "HTR-W1-P2-PACKED-1", "L": 0, "K": 2, "experts": [Boom()]}, f)
+    with pytest.raises(Exception) as ei:
+        checkpoint.read_packed_chunk(str(tmp_path / "evil.pt"))
+    assert "Unsupported" in str(ei.value) or "weights_only" in str(ei.value) or "pickle" in str(ei.value).lower()

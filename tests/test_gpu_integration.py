@@ -275,3 +275,35 @@ def test_captures_own_their_workspaces(dev):
         torch.cuda.synchronize()
         assert torch.equal(y1, want) and torch.equal(y2, want)
     del filler
+
+
+def test_packed_expert_chunks_feed_the_grouped_launch(dev, oracle):
+    """The committed routed-expert chunks (reference layout, htr/moe_encode.py:216-225; four experts, K3) are read with
+    the weights-only loader, fused to gate_up / down lists and run through ops.moe_experts; the result is compared with
+    the per-expert composition on the CPU oracle, and every decoded matrix with the oracle's float64 decode."""
+    import os
+    from htr_amd import checkpoint, ops
+    print("packed expert chunks -> moe_experts", flush=True)
+    root = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "moe_L3")
+    gate_up, down, K = checkpoint.PackedExperts(root).layer(3, device=dev)
+    E, T, TOP, H, F = 4, 12, 2, 256, 128
+    for e in range(E):
+        for t in (gate_up[e], down[e]):
+            W = ops.dequant_w(*t).float().cpu().numpy()
+            W_ref = oracle.np_dequant_w(*[v.cpu().numpy() for v in t])
+            assert np.abs(W - W_ref).max() <= 2.0 ** -8 * np.abs(W_ref).max()          # bf16 output
+    g = torch.Generator().manual_seed(31)
+    w, ids = torch.topk(torch.softmax(torch.randn(T, E, generator=g), dim=-1), TOP, dim=-1)
+    x = torch.randn(T, H, generator=g).bfloat16()
+    y = ops.moe_experts(x.to(dev), ids.to(dev), w.to(dev), gate_up, down).cpu().numpy()
+    y_ref = np.zeros((T, H))
+    for e in range(E):
+        tok, slot = torch.nonzero(ids == e, as_tuple=True)
+        if tok.numel() == 0:
+            continue
+        r2 = torch.from_numpy(oracle.c_linear(x[tok].float().numpy(), *[v.cpu().numpy() for v in gate_up[e]])).float()
+        rh = (torch.nn.functional.silu(r2[:, :F]) * r2[:, F:]).bfloat16().float().numpy()
+        ro = oracle.c_linear(rh, *[v.cpu().numpy() for v in down[e]])
+        np.add.at(y_ref, tok.numpy(), ro * w[tok, slot].numpy().astype(np.float64)[:, None])
+    rel = np.abs(y - y_ref).max() / np.abs(y_ref).max()
+    assert rel <= 4e-3, rel          # two chained linears with a bf16 rounding between them

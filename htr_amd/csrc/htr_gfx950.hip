@@ -1579,7 +1579,7 @@ __global__ __launch_bounds__(512) void k_dequant_w(const uint32_t* __restrict__ 
 // the first index among equal values in every min / argmin.
 template <int K> struct VitCfg {
   static constexpr int NB = 1 << K, SJ = 65536 >> K;
-  static constexpr int THREADS = K == 2 ? 1024 : 512;
+  static constexpr int THREADS = K == 2 ? 1024 : (K == 8 ? 256 : 512);   // at most one thread per M entry
   static constexpr int ITEMS = SJ / THREADS;         // M entries per thread
 };
 
@@ -2230,14 +2230,14 @@ int htr_linear_grouped(const htr_group_entry* entries, int count, int m, int n, 
 }
 
 size_t htr_viterbi_workspace_bytes(int64_t tiles, int T, int K) {
-  if (tiles <= 0 || T < 1 || T > 256 || K < 2 || K > 7) return 0;
+  if (tiles <= 0 || T < 1 || T > 256 || K < 2 || K > 8) return 0;
   return align256((size_t)tiles * (size_t)(T > 1 ? T - 1 : 1) * (65536u >> K));
 }
 
 int htr_viterbi(const void* x, const void* w, int64_t tiles, int T, int K, int tailbite, void* states_u16, void* workspace,
                 size_t workspace_bytes, void* stream) {
   if (!x || !w || !states_u16) return HTR_ERR_NULL;
-  if (K < 2 || K > 7) return HTR_ERR_K;
+  if (K < 2 || K > 8) return HTR_ERR_K;
   if (tiles <= 0 || tiles > 0x7FFFFFFF || T < 1 || T > 256) return HTR_ERR_SHAPE;
   if (((uintptr_t)x & 3) || ((uintptr_t)w & 3) || ((uintptr_t)states_u16 & 1)) return HTR_ERR_ALIGN;
   const size_t need = htr_viterbi_workspace_bytes(tiles, T, K);
@@ -2257,7 +2257,8 @@ int htr_viterbi(const void* x, const void* w, int64_t tiles, int T, int K, int t
     case 4: HTR_LAUNCH_VIT(4); break;
     case 5: HTR_LAUNCH_VIT(5); break;
     case 6: HTR_LAUNCH_VIT(6); break;
-    default: HTR_LAUNCH_VIT(7); break;
+    case 7: HTR_LAUNCH_VIT(7); break;
+    default: HTR_LAUNCH_VIT(8); break;
   }
 #undef HTR_LAUNCH_VIT
   return HTR_OK;

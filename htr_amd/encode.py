@@ -16,16 +16,24 @@ VITERBI = None
 # tiles per launch: bounds the backpointer scratch (tiles * 255 * (65536 >> K) bytes)
 MAX_SCRATCH_BYTES = 1 << 30
 _SCRATCH = {}
+_CHECKED_CB = set()          # data pointers of codebook tensors already compared with the procedural codebook
 
 
 def viterbi(x, w, cb=None, K=4, tailbite=True):
     """Tail-biting bitshift-trellis Viterbi on the GPU (htr.reference.viterbi / htr.vit_v2.viterbi of the reference).
 
     x, w: float32 [B, T <= 256] on a ROCm device.  cb is accepted for signature compatibility and must be the HTR
-    codebook (the kernel evaluates it procedurally).  Returns int64 states [B, T].
+    codebook (the kernel evaluates it procedurally; another table is refused).  Returns int64 states [B, T].
+    Costs that are NaN never win a comparison in the kernel, where torch.argmin in the reference returns the first NaN:
+    inputs with NaN give different (meaningless either way) states.
     """
     if not x.is_cuda:
-        raise RuntimeError("htr_amd.encode.viterbi runs on a ROCm device only")
+        raise RuntimeError("htr_amd.encode.viterbi runs on a ROCm device only; for CPU tensors set encode.VITERBI to a "
+                           "CPU search with the signature (x, w, cb, K) -> states")
+    if cb is not None and cb.data_ptr() not in _CHECKED_CB:
+        if cb.numel() != wire.S or not torch.equal(cb.detach().float().cpu().reshape(-1), wire.codebook_f32("cpu")):
+            raise RuntimeError("viterbi: cb is not the HTR-W1 codebook; the GPU search evaluates that codebook only")
+        _CHECKED_CB.add(cb.data_ptr())
     x = x.float().contiguous()
     w = w.float().contiguous()
     B, T = x.shape
@@ -34,7 +42,7 @@ def viterbi(x, w, cb=None, K=4, tailbite=True):
     L = _native.lib()
     per_tile = L.htr_viterbi_workspace_bytes(1, T, K)
     if per_tile == 0:
-        raise RuntimeError(f"viterbi: unsupported K {K} (2..7)")
+        raise RuntimeError(f"viterbi: unsupported K {K} (2..8)")
     out = torch.empty((B, T), dtype=torch.int16, device=x.device)
     batch = max(1, min(B, MAX_SCRATCH_BYTES // per_tile))
     cus = torch.cuda.get_device_properties(x.device).multi_processor_count
@@ -56,9 +64,15 @@ def viterbi(x, w, cb=None, K=4, tailbite=True):
 
 
 def block_rotate(W, bs=wire.RHT_BLOCK):
-    """Blocks of bs columns times H^T (H is symmetric; kept as in htr/encode.py:15-17)."""
+    """Blocks of bs columns times H^T (H is symmetric; htr/encode.py:15-17)."""
     m, n = W.shape
     return (W.reshape(m, n // bs, bs) @ wire.hadamard(bs, W.device).T).reshape(m, n)
+
+
+def _rotate_both_sides(A, row_signs, col_signs):
+    """diag(row_signs) A diag(col_signs) with the blockwise Hadamard applied to its columns, then to its rows."""
+    B = block_rotate(A * row_signs[:, None] * col_signs[None, :])
+    return block_rotate(B.T.contiguous()).T
 
 
 def make_signs(n, m, seed, index, shared_su):
@@ -88,75 +102,94 @@ def prep_H(H, W, damp=0.01):
     return H, W
 
 
-class _Job:
-    """One matrix of an input group in the rotated basis."""
+def _feedback_factor(Hd):
+    """Block LDL feedback matrix of a damped, rotated Hessian (float64 in, float32 out): the Cholesky factor with every
+    16-column block normalised by its own 16x16 diagonal block (htr/encode.py:64-67)."""
+    n = Hd.shape[0]
+    nb = n // 16
+    C = torch.linalg.cholesky(Hd)
+    diag_blocks = C.view(nb, 16, nb, 16).diagonal(dim1=0, dim2=2).permute(2, 0, 1)
+    return torch.einsum("ikj,kjl->ikl", C.view(n, nb, 16), torch.linalg.inv(diag_blocks)).reshape(n, n).float()
 
-    def __init__(self, W, H, su, sv, damp):
-        n = W.shape[1]
-        nb = n // 16
-        Wt = block_rotate(W * sv[:, None] * su[None, :])
-        Wt = block_rotate(Wt.T.contiguous()).T
-        Ht = block_rotate(H * su[:, None] * su[None, :])
-        Ht = block_rotate(Ht.T.contiguous()).T.contiguous()
-        Ht, Wt = prep_H(Ht, Wt.contiguous(), damp)
-        self.rs = Wt.pow(2).mean(dim=1).sqrt().half().float().clamp(min=1e-8)      # row scales, as stored (fp16)
-        # block LDL feedback matrix: C = chol(H), normalised by its 16x16 diagonal blocks
-        C = torch.linalg.cholesky(Ht)
-        diag = C.view(nb, 16, nb, 16).diagonal(dim1=0, dim2=2).permute(2, 0, 1)
-        self.Lb = torch.einsum("ikj,kjl->ikl", C.view(n, nb, 16), torch.linalg.inv(diag)).reshape(n, n).float()
-        self.Wt = Wt.float()
-        self.su, self.sv = su, sv
+
+class _Group:
+    """The matrices of one input group in the rotated basis, stacked along the rows: every 16-column block of the whole
+    group is one batch of 256-weight tiles for the search (one workgroup per tile on the GPU), and matrices that came
+    with the same Hessian (gate and up of an expert, q / k / v of a layer) share one factorisation and one feedback
+    product."""
+
+    def __init__(self, jobs, seed, shared_su, damp):
+        n = jobs[0]["W"].shape[1]
+        if n % 128:
+            raise RuntimeError("encode_group: n must be a multiple of 128")
+        self.n, self.nb = n, n // 16
+        dev = jobs[0]["W"].device
+        self.signs, self.rows = [], []            # (su, sv) and the row range of every matrix in the stack
+        self.factors = []                         # [first row, last row, feedback matrix]: consecutive matrices of one Hessian
+        Wt, seen = [], {}
+        r0 = 0
+        for index, jb in enumerate(jobs):
+            W = jb["W"].float()
+            m = W.shape[0]
+            if m % 128 or W.shape[1] != n:
+                raise RuntimeError("encode_group: every matrix needs m % 128 == 0 and the group's n")
+            su, sv = (s.to(W.device) for s in make_signs(n, m, seed, index, shared_su))
+            Hr = _rotate_both_sides(jb["H"].float().to(W.device), su, su).contiguous()
+            Hd, Wr = prep_H(Hr, _rotate_both_sides(W, sv, su).contiguous(), damp)
+            Wt.append(Wr.float())
+            # the damped Hessian depends on (H, su) only: the same H object under a shared su is factored once
+            key = id(jb["H"]) if shared_su else None
+            if key is not None and key in seen and self.factors[-1][2] is seen[key]:
+                self.factors[-1][1] = r0 + m
+            else:
+                Lb = seen.get(key) if key is not None else None
+                if Lb is None:
+                    Lb = _feedback_factor(Hd)
+                    if key is not None:
+                        seen[key] = Lb
+                self.factors.append([r0, r0 + m, Lb])
+            self.signs.append((su, sv))
+            self.rows.append((r0, r0 + m))
+            r0 += m
+        self.Wt = torch.cat(Wt)
+        self.rs = self.Wt.pow(2).mean(dim=1).sqrt().half().float().clamp(min=1e-8)      # row scales, as stored (fp16)
         self.Q = torch.zeros_like(self.Wt)
-        self.F = torch.zeros_like(self.Wt)
-        self.S = torch.zeros((W.shape[0] // 16, nb, 256), dtype=torch.int64, device=W.device)
+        self.F = torch.zeros_like(self.Wt)                                              # error fed forward
+        self.S = torch.zeros((r0 // 16, self.nb, 256), dtype=torch.int64, device=dev)
+        # search weights: the squared row scales of a tile's 16 rows, normalised to mean 1 per tile; the same for every block
+        wg = (self.rs[:, None] ** 2).expand(-1, 16).contiguous().reshape(-1, 256)
+        self.wg = wg / wg.mean(dim=1, keepdim=True)
 
 
 @torch.no_grad()
 def encode_group(jobs, K, seed=1234, shared_su=True, damp=0.01, max_batch=1024, log=None):
     """jobs: list of dict(W=[m, n], H=[n, n]) sharing n.  Returns a list of dict(qweight, scales, su, sv, What, Q)
-    (htr/encode.py:45-110)."""
+    (htr/encode.py:45-110): block LDLQ from the last 16-column block to the first, each block's tiles quantized by the
+    trellis search against the row scales, the block's error fed forward through the feedback matrix."""
     search = VITERBI or (lambda x, w, cb, k: viterbi(x, w, cb, k))
-    n = jobs[0]["W"].shape[1]
-    if n % 128:
-        raise RuntimeError("encode_group: n must be a multiple of 128")
-    nb = n // 16
-    dev = jobs[0]["W"].device
-    cb = wire.codebook_f32(dev)
-    P = []
-    for index, jb in enumerate(jobs):
-        W = jb["W"].float()
-        if W.shape[0] % 128 or W.shape[1] != n:
-            raise RuntimeError("encode_group: every matrix needs m % 128 == 0 and the group's n")
-        su, sv = make_signs(n, W.shape[0], seed, index, shared_su)
-        P.append(_Job(W, jb["H"].float().to(W.device), su.to(W.device), sv.to(W.device), damp))
-    for k in range(nb - 1, -1, -1):                     # 16-column blocks, last first
+    G = _Group(jobs, seed, shared_su, damp)
+    cb = wire.codebook_f32(G.Wt.device)
+    ntiles = G.wg.shape[0]
+    for k in range(G.nb - 1, -1, -1):
         cols = slice(16 * k, 16 * k + 16)
-        X = torch.cat([((p.Wt[:, cols] + p.F[:, cols]) / p.rs[:, None]).reshape(-1, 256) for p in P])
-        Wg = torch.cat([(p.rs[:, None] ** 2).expand(-1, 16).contiguous().reshape(-1, 256) for p in P])
-        Wg = Wg / Wg.mean(dim=1, keepdim=True)
-        ST = torch.empty(X.shape, dtype=torch.int64, device=X.device)
-        for b0 in range(0, X.shape[0], max_batch):
-            ST[b0:b0 + max_batch] = search(X[b0:b0 + max_batch].contiguous(), Wg[b0:b0 + max_batch].contiguous(), cb, K)
-        R = cb[ST]
-        off = 0
-        for p in P:
-            m = p.Wt.shape[0]
-            nt = m // 16
-            p.S[:, k] = ST[off:off + nt]
-            q = R[off:off + nt].reshape(m, 16) * p.rs[:, None]
-            off += nt
-            p.Q[:, cols] = q
-            if k > 0:
-                p.F[:, :16 * k] += (p.Wt[:, cols] - q) @ p.Lb[cols, :16 * k]
+        target = ((G.Wt[:, cols] + G.F[:, cols]) / G.rs[:, None]).reshape(-1, 256)
+        for b0 in range(0, ntiles, max_batch):
+            G.S[b0:b0 + max_batch, k] = search(target[b0:b0 + max_batch].contiguous(), G.wg[b0:b0 + max_batch].contiguous(), cb, K)
+        q = cb[G.S[:, k]].reshape(-1, 16) * G.rs[:, None]
+        G.Q[:, cols] = q
+        if k > 0:
+            err = G.Wt[:, cols] - q
+            for first, last, Lb in G.factors:
+                G.F[first:last, :16 * k] += err[first:last] @ Lb[cols, :16 * k]
         if log and k % 32 == 0:
-            log(f"  block {k}/{nb}")
+            log(f"  block {k}/{G.nb}")
     outs = []
-    for p in P:
-        mt = p.S.shape[0]
-        qweight = wire.pack_states(p.S.reshape(-1, 256), K).reshape(mt, nb, 8 * K)
-        W = wire.blk_had_cols_T(p.Q.T.contiguous()).T
-        W = wire.blk_had_cols_T(W.contiguous())
-        What = (W * p.sv[:, None] * p.su[None, :]).contiguous()
-        outs.append(dict(qweight=qweight.cpu(), scales=p.rs.half().cpu(), su=wire.pack_signs(p.su).cpu(),
-                         sv=wire.pack_signs(p.sv).cpu(), What=What, Q=p.Q))
+    for (first, last), (su, sv) in zip(G.rows, G.signs):
+        Q = G.Q[first:last]
+        S = G.S[first // 16:last // 16]
+        qweight = wire.pack_states(S.reshape(-1, 256), K).reshape(S.shape[0], G.nb, 8 * K)
+        W = wire.blk_had_cols_T(wire.blk_had_cols_T(Q.T.contiguous()).T.contiguous())
+        What = (W * sv[:, None] * su[None, :]).contiguous()
+        outs.append(dict(qweight=qweight.cpu(), scales=G.rs[first:last].half().cpu(), su=wire.pack_signs(su).cpu(),
+                         sv=wire.pack_signs(sv).cpu(), What=What, Q=Q))
     return outs

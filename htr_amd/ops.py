@@ -16,7 +16,8 @@ _DTYPE_CODE = {torch.bfloat16: _native.BF16, torch.float16: _native.F16, torch.f
 
 # One launch takes up to this many activation rows; longer inputs are cut into chunks that each
 # re-read the packed weight (the reference does the same in 8-row chunks, htr/ops.py:77-88).
-LAUNCH_MAX_M = _native.MAX_BATCH
+# HTR_GEMV_MAX_M lowers it (the reference's knob of that name is its rows per decode launch, 8 there: htr/ops.py:48).
+LAUNCH_MAX_M = max(1, min(_native.MAX_BATCH, int(os.environ.get("HTR_GEMV_MAX_M", str(_native.MAX_BATCH)))))
 GROUP_MAX_M = _native.MAX_GROUP_ROWS      # rows per entry of a grouped launch
 # explicit chunk length (steps per workgroup) for experiments; 0 = library policy
 NSPLIT = int(os.environ.get("HTR_NSPLIT", "0"))
@@ -26,6 +27,11 @@ NSPLIT = int(os.environ.get("HTR_NSPLIT", "0"))
 # Measured on MI355X (K4): one fused launch of 128 rows takes 32 / 42 / 59 us on 4096x4096 / 14336x4096 / 4096x14336,
 # dequantize + GEMM 42 / 73 / 105 us; two fused launches (256 rows) no longer beat it.
 GEMV_LOOP_MAX = int(os.environ.get("HTR_GEMV_LOOP_MAX", "128"))
+# How inputs beyond GEMV_LOOP_MAX rows are multiplied (the reference's HTR_PREFILL, htr/ops.py:52-54): "w" = dequantize
+# to the original basis and one library GEMM (default); "rot" = stay in the rotated basis: rotate the activations, GEMM
+# against the dequantized Q, rotate the result (the reference's slower first-version path, htr/ops.py:101-104; here
+# with float32 Q from htr_dequant_q and torch products, kept for cross-checks).
+PREFILL = os.environ.get("HTR_PREFILL", "w")
 
 class _Workspace:
     """One device buffer for split partials and pre-rotated activations, with its failure flag in pinned host memory."""
@@ -142,7 +148,15 @@ def _linear_impl(x2, qweight, scales, su, sv, bias, out_dtype=None):
             raise RuntimeError("HTR-W1 tensors must be contiguous and on the device of x")
     if bias is not None and (bias.dtype != out_dtype or bias.numel() != m or bias.device != x2.device):
         raise RuntimeError("bias must be [m] in the output dtype on the device of x")
+    if M > GEMV_LOOP_MAX and PREFILL == "rot":
+        xr = wire.blk_had_cols_T(x2.float() * wire.unpack_signs(su, n).to(x2.device))
+        yr = wire.blk_had_cols_T(xr @ dequant_q(qweight, scales).T) * wire.unpack_signs(sv, m).to(x2.device)
+        if bias is not None:
+            yr = yr + bias.float()
+        return yr.to(out_dtype)
     if M > GEMV_LOOP_MAX:
+        if PREFILL != "w":
+            raise RuntimeError(f"HTR_PREFILL = {PREFILL!r}: expected 'w' or 'rot'")
         W = dequant_w(qweight, scales, su, sv)
         if x2.dtype != torch.bfloat16:
             W = W.to(x2.dtype)

@@ -9,6 +9,7 @@ environment), minimal stand-ins for the four vLLM names are used so that the sel
 exercised; `register()` refuses to run without the real package.
 """
 import collections
+import itertools
 import json
 import os
 import time
@@ -53,15 +54,12 @@ except ImportError:
 
 # module-name fragments that are never quantized (vision / audio towers, multi-token-prediction heads)
 SKIP = ("visual", "vision", "audio", "mtp")
-_QKV_INDEX = {"q": 0, "k": 1, "v": 2}
 
 
 def canon(name):
     """Checkpoint/module name -> key of the `modules` table: no ".weight" suffix, path from the last "layers." on."""
-    if name.endswith(".weight"):
-        name = name[:-len(".weight")]
-    at = name.rfind("layers.")
-    return name if at < 0 else name[at:]
+    _, marker, tail = name.removesuffix(".weight").rpartition("layers.")
+    return marker + tail
 
 
 @register_quantization_config("htr")
@@ -92,45 +90,101 @@ class HTRConfig(QuantizationConfig):
     def from_config(cls, config):
         return cls(config.get("modules", {}), config.get("wire", "HTR-W1"))
 
+    def _width(self, prefix):
+        """Bit width of the module at `prefix`, or None if the checkpoint does not quantize it.  A module that the
+        model fuses from several checkpoint modules (packed_modules_mapping: qkv_proj <- q_proj, k_proj, v_proj) is
+        looked up part by part: all parts quantized at one width, or none."""
+        scope, dot, leaf = canon(prefix).rpartition(".")
+        parts = (getattr(self, "packed_modules_mapping", None) or {}).get(leaf, [leaf])
+        found = {part: self.modules.get(scope + dot + part) for part in parts}
+        widths = set(found.values())
+        if widths == {None}:
+            return None
+        if len(widths) > 1:
+            raise ValueError(f"HTR: fused module {prefix} has mixed quantization {found}")
+        return widths.pop()
+
     def get_quant_method(self, layer, prefix):
-        parts = prefix.split(".")
         if isinstance(layer, ParallelLMHead):
             # only an output head named lm_head that the checkpoint lists; other embeddings stay unquantized
-            K = self.modules.get("lm_head")
-            return HTRLinearMethod(K) if K is not None and parts[-1] == "lm_head" else None
+            K = self.modules.get("lm_head") if prefix.split(".")[-1] == "lm_head" else None
+            return None if K is None else HTRLinearMethod(K)
         if not isinstance(layer, LinearBase):
             return None
-        if any(tag in parts or tag in prefix for tag in SKIP):
-            return UnquantizedLinearMethod()
-        key = canon(prefix)
-        parent, _, leaf = key.rpartition(".")
-        packed = getattr(self, "packed_modules_mapping", None) or {}
-        members = packed.get(leaf, [leaf])
-        widths = [self.modules.get(f"{parent}.{name}" if parent else name) for name in members]
-        if all(k is None for k in widths):
-            return UnquantizedLinearMethod()
-        if None in widths or len(set(widths)) != 1:
-            raise ValueError(f"HTR: fused module {prefix} has mixed quantization {dict(zip(members, widths))}")
-        return HTRLinearMethod(widths[0])
+        in_skipped_tower = any(tag in prefix for tag in SKIP)
+        K = None if in_skipped_tower else self._width(prefix)
+        return UnquantizedLinearMethod() if K is None else HTRLinearMethod(K)
+
+
+class _FusedRows:
+    """Output-row layout of a module stacked from several parts (q | k | v, gate | up): which rows a checkpoint shard
+    covers.  A shard is named by part index, by "q" / "k" / "v", by a run of consecutive part indices, or not at all
+    (the whole module)."""
+    NAMED = {"q": 0, "k": 1, "v": 2}
+
+    def __init__(self, sizes):
+        self.edges = list(itertools.accumulate(sizes, initial=0))      # part i covers rows edges[i] .. edges[i + 1]
+
+    def rows(self, shard_id):
+        last = len(self.edges) - 2
+        if shard_id is None:
+            lo, hi = 0, last
+        elif isinstance(shard_id, (tuple, list)):
+            lo, hi = shard_id[0], shard_id[-1]
+            assert list(shard_id) == list(range(lo, hi + 1)), f"shard {shard_id} is not a run of consecutive parts"
+        else:
+            lo = hi = self.NAMED[shard_id] if isinstance(shard_id, str) else int(shard_id)
+        assert 0 <= lo <= hi <= last, (shard_id, last)
+        return self.edges[lo], self.edges[hi + 1]
+
+    def span(self, shard_id, unit):
+        """(first, count) of the shard in entries of `unit` output rows each."""
+        r0, r1 = self.rows(shard_id)
+        assert r0 % unit == 0 and r1 % unit == 0, (r0, r1, unit)
+        return r0 // unit, (r1 - r0) // unit
 
 
 def _shard_range(sizes, shard_id, unit):
-    """(first, count) in `unit`-row units of the output rows that `shard_id` covers in a fused module."""
-    if shard_id is None:
-        picked = list(range(len(sizes)))
-    elif isinstance(shard_id, str):
-        picked = [_QKV_INDEX[shard_id]]
-    elif isinstance(shard_id, (tuple, list)):
-        picked = list(shard_id)
-    else:
-        picked = [int(shard_id)]
-    if picked != list(range(picked[0], picked[-1] + 1)):
-        raise AssertionError(picked)
-    first = sum(sizes[:picked[0]])
-    count = sum(sizes[i] for i in picked)
-    if first % unit or count % unit:
-        raise AssertionError((first, count, unit))
-    return first // unit, count // unit
+    return _FusedRows(sizes).span(shard_id, unit)
+
+
+class _RowPlacer:
+    """weight_loader of a tensor indexed by output rows: a shard lands at its row offset, in the tensor's own unit."""
+
+    def __init__(self, layout, unit):
+        self.layout, self.unit = layout, unit
+
+    def __call__(self, param, loaded, shard_id=None):
+        if shard_id is None:
+            shard_id = getattr(loaded, "shard_id", None)               # stacked-parameter mappers attach it to the tensor
+        first, count = self.layout.span(shard_id, self.unit)
+        dest = param.data.narrow(0, first, count)
+        assert dest.shape == loaded.shape, (tuple(param.shape), tuple(loaded.shape), shard_id)
+        dest.copy_(loaded)
+
+
+class _SharedSigns:
+    """weight_loader of the input sign vector: every part of a fused module brings the same one (docs/FORMAT.md:31-32);
+    the first is kept, the others are compared with it."""
+
+    def __init__(self):
+        self.filled = False
+
+    def __call__(self, param, loaded, shard_id=None):
+        assert loaded.shape == param.shape
+        if self.filled and not torch.equal(param.data.cpu(), loaded.cpu()):
+            raise ValueError("HTR: fused shards do not share the input sign vector")
+        if not self.filled:
+            param.data.copy_(loaded)
+            self.filled = True
+
+
+# tensors indexed by output rows: name -> (dtype, output rows per entry of dim 0, trailing dims for n inputs at width K)
+_ROW_TENSORS = {
+    "htr_qweight": (torch.int32, 16, lambda n, K: (n // 16, 8 * K)),
+    "htr_scales": (torch.float16, 1, lambda n, K: ()),
+    "htr_sv": (torch.uint8, 8, lambda n, K: ()),
+}
 
 
 class HTRLinearMethod(LinearMethodBase):
@@ -142,43 +196,20 @@ class HTRLinearMethod(LinearMethodBase):
     def create_weights(self, layer, input_size_per_partition, output_partition_sizes, input_size, output_size,
                        params_dtype, **extra_weight_attrs):
         n, sizes = input_size_per_partition, list(output_partition_sizes)
-        m = sum(sizes)
-        assert input_size_per_partition == input_size, "HTR: tensor parallelism is not supported"
+        assert n == input_size, "HTR: tensor parallelism is not supported"
         assert n % 128 == 0 and all(s % 128 == 0 for s in sizes), (n, sizes)
-        K = self.K
-        tensors = {
-            "htr_qweight": torch.empty(m // 16, n // 16, 8 * K, dtype=torch.int32),
-            "htr_scales": torch.empty(m, dtype=torch.float16),
-            "htr_su": torch.empty(n // 8, dtype=torch.uint8),
-            "htr_sv": torch.empty(m // 8, dtype=torch.uint8),
-        }
+        layout = _FusedRows(sizes)
+        m = layout.edges[-1]
 
-        def row_loader(unit):
-            # qweight rows are 16 output rows, scales 1, sv 8: a fused shard lands at its row offset in those units
-            def load(param, loaded, shard_id=None):
-                if shard_id is None:
-                    shard_id = getattr(loaded, "shard_id", None)      # stacked-parameter mappers attach it to the tensor
-                first, count = _shard_range(sizes, shard_id, unit)
-                assert tuple(loaded.shape) == (count,) + tuple(param.shape[1:]), (param.shape, loaded.shape, shard_id)
-                param.data[first:first + count].copy_(loaded)
-            return load
-
-        def su_loader(param, loaded, shard_id=None):
-            # the parts of a fused module must share the input sign vector (docs/FORMAT.md:31-32)
-            assert loaded.shape == param.shape
-            if getattr(param, "_htr_loaded", False):
-                if not torch.equal(param.data.cpu(), loaded.cpu()):
-                    raise ValueError("HTR: fused shards do not share the input sign vector")
-                return
-            param.data.copy_(loaded)
-            param._htr_loaded = True
-
-        loaders = {"htr_qweight": row_loader(16), "htr_scales": row_loader(1), "htr_sv": row_loader(8), "htr_su": su_loader}
-        for name, value in tensors.items():
-            p = Parameter(value, requires_grad=False)
+        def attach(name, tensor, loader):
+            p = Parameter(tensor, requires_grad=False)
             layer.register_parameter(name, p)
-            set_weight_attrs(p, {"weight_loader": loaders[name]})
-        layer.htr_K = K
+            set_weight_attrs(p, {"weight_loader": loader})
+
+        for name, (dtype, unit, trailing) in _ROW_TENSORS.items():
+            attach(name, torch.empty((m // unit,) + trailing(n, self.K), dtype=dtype), _RowPlacer(layout, unit))
+        attach("htr_su", torch.empty(n // 8, dtype=torch.uint8), _SharedSigns())
+        layer.htr_K = self.K
 
     def process_weights_after_loading(self, layer):
         pass
@@ -186,29 +217,37 @@ class HTRLinearMethod(LinearMethodBase):
     def apply(self, layer, x, bias=None):
         from . import ops
         if _COUNT_FILE is not None:
-            _census(x, layer.htr_K)
+            _CENSUS.note(x.numel() // x.shape[-1], layer.htr_K)
         return ops.linear(x, layer.htr_qweight, layer.htr_scales, layer.htr_su, layer.htr_sv, bias)
 
 
-# ---- dispatch census (HTR_COUNT_FILE): calls per batch bucket and per K, dumped atomically every 512 calls
+# ---- dispatch census (HTR_COUNT_FILE=<path>): calls per batch bucket ("M1", "M2-8", "M>8") and per bit width ("K4"),
+# written to <path>.<pid>.json every 512 calls through a temporary file and a rename
 _COUNT_FILE = os.environ.get("HTR_COUNT_FILE") or None
-_COUNTS = collections.Counter()
-_BUCKETS = ("M1", "M2-8", "M>8")
 
 
-def _census(x, K):
-    M = x.numel() // x.shape[-1]
-    _COUNTS[_BUCKETS[0] if M == 1 else (_BUCKETS[1] if M <= 8 else _BUCKETS[2])] += 1
-    _COUNTS["K%d" % K] += 1
-    if sum(_COUNTS[b] for b in _BUCKETS) % 512 == 0:
-        _dump_counts()
+class _Census:
+    EVERY = 512
+
+    def __init__(self):
+        self.counts = collections.Counter()
+        self.calls = 0
+
+    def note(self, rows, K):
+        self.counts["M1" if rows == 1 else "M2-8" if rows <= 8 else "M>8"] += 1
+        self.counts[f"K{K}"] += 1
+        self.calls += 1
+        if self.calls % self.EVERY == 0:
+            self.dump()
+
+    def dump(self):
+        final = f"{_COUNT_FILE}.{os.getpid()}.json"
+        with open(final[:-5] + ".tmp", "w") as f:
+            json.dump({"pid": os.getpid(), "t": time.time(), "counts": dict(self.counts)}, f)
+        os.replace(final[:-5] + ".tmp", final)
 
 
-def _dump_counts():
-    tmp = f"{_COUNT_FILE}.{os.getpid()}.tmp"
-    with open(tmp, "w") as f:
-        json.dump(dict(pid=os.getpid(), t=time.time(), counts=dict(_COUNTS)), f)
-    os.replace(tmp, f"{_COUNT_FILE}.{os.getpid()}.json")
+_CENSUS = _Census()
 
 
 def register():

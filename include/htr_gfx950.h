@@ -187,7 +187,7 @@ void htr_set_spin_limit(int polls);
  *   x, w      float32 [tiles, T] targets and per-element weights (T <= 256; the codec uses 256)
  *   states    uint16 [tiles, T]: s_t with s_t >> K == s_{t-1} & (2^(16-K) - 1), circular when tailbite != 0
  *   workspace htr_viterbi_workspace_bytes() bytes of device scratch (backpointers; no zero requirement)
- * K = 2..7.  Same result as the reference's portable search, htr.reference.viterbi(x, w, codebook_f32(), K)
+ * K = 2..8.  Same result as the reference's portable search, htr.reference.viterbi(x, w, codebook_f32(), K)
  * (htr/reference.py:6-50), which its CUDA versions htr/vit_v1.py:46-110 and htr/vit_v2.py:100-162 also reproduce;
  * the state values are the procedural codebook, so no codebook tensor is passed.
  */

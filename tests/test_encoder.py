@@ -60,6 +60,23 @@ def test_encoder_reproduces_reference_with_hessian_and_shared_signs(oracle_searc
     assert np.array_equal(rs[0]["su"].numpy(), rs[1]["su"].numpy())          # one input sign vector for the group
 
 
+def test_matrices_of_one_hessian_share_a_factorisation(oracle_search, enc_gold, monkeypatch):
+    """Two matrices that come with the same Hessian object under a shared input sign vector are factored once and fed
+    back with one product; the result is the one of separate factorisations (the reference's fixture)."""
+    calls = []
+    real = oracle_search._feedback_factor
+    monkeypatch.setattr(oracle_search, "_feedback_factor", lambda Hd: (calls.append(1), real(Hd))[1])
+    H = torch.from_numpy(enc_gold["b_H"])
+    jobs = [{"W": torch.from_numpy(enc_gold[f"b{i}_W"]), "H": H} for i in range(2)]
+    rs = oracle_search.encode_group(jobs, 3, seed=4321, max_batch=64)
+    assert len(calls) == 1
+    for i, r in enumerate(rs):
+        assert np.array_equal(r["qweight"].numpy(), enc_gold[f"b{i}_qweight"])
+    calls.clear()
+    oracle_search.encode_group([{"W": jobs[0]["W"], "H": H}, {"W": jobs[1]["W"], "H": H.clone()}], 3, seed=4321, max_batch=64)
+    assert len(calls) == 2
+
+
 def test_sign_draws_and_hessian_preparation():
     from htr_amd import encode
     su, sv = encode.make_signs(256, 128, 99, 2, True)
@@ -99,7 +116,8 @@ def test_gpu_search_matches_reference_vectors(dev, vit_gold, K):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("K,B,T,tailbite", [(2, 5, 256, True), (3, 7, 256, True), (4, 9, 256, True), (5, 6, 256, True),
-                                            (6, 3, 256, True), (7, 2, 256, True), (4, 3, 256, False), (3, 4, 100, True),
+                                            (6, 3, 256, True), (7, 2, 256, True), (8, 3, 256, True), (8, 2, 256, False), (8, 2, 9, True),
+                                            (4, 3, 256, False), (3, 4, 100, True),
                                             (4, 2, 1, True), (2, 2, 17, False)])
 def test_gpu_search_matches_oracle(dev, oracle, K, B, T, tailbite):
     from htr_amd import encode
@@ -111,6 +129,19 @@ def test_gpu_search_matches_oracle(dev, oracle, K, B, T, tailbite):
     st = encode.viterbi(x.to(dev), w.to(dev), None, K, tailbite=tailbite).cpu().numpy()
     want = oracle.c_viterbi(x.numpy(), w.numpy(), K, tailbite=tailbite)
     assert np.array_equal(st.astype(np.uint32), want)
+
+
+@pytest.mark.gpu
+def test_gpu_search_refuses_another_codebook_and_cpu_tensors(dev):
+    from htr_amd import encode, wire
+    print("viterbi: codebook check", flush=True)
+    x, w = torch.zeros(1, 16), torch.ones(1, 16)
+    cb = wire.codebook_f32(dev)
+    assert encode.viterbi(x.to(dev), w.to(dev), cb, 4).shape == (1, 16)
+    with pytest.raises(RuntimeError, match="not the HTR-W1 codebook"):
+        encode.viterbi(x.to(dev), w.to(dev), cb * 2.0, 4)
+    with pytest.raises(RuntimeError, match="set encode.VITERBI"):
+        encode.viterbi(x, w, None, 4)
 
 
 @pytest.mark.gpu

@@ -106,6 +106,29 @@ def test_prefill_path_dequant_then_gemm(dev, oracle):
     assert _rel(y.float().cpu().numpy(), ref) <= 2.0 ** -6
 
 
+def test_reference_env_knobs(dev, oracle, monkeypatch):
+    """The reference's HTR_PREFILL = "rot" (rotated-basis GEMM, htr/ops.py:52-54, 101-104) and HTR_GEMV_MAX_M (rows per
+    decode launch, htr/ops.py:48) as module settings: same results as the default paths."""
+    from htr_amd import ops
+    print("env knobs: prefill rot, rows per launch", flush=True)
+    qw, sc, su, sv, x = _case(512, 384, 4, 160, 809)
+    bias = torch.randn(512, generator=torch.Generator().manual_seed(3)).bfloat16()
+    d = [t.to(dev) for t in (qw, sc, su, sv)]
+    ref = _ref(oracle, qw, sc, su, sv, x, bias)
+    monkeypatch.setattr(ops, "PREFILL", "rot")
+    y = ops.linear(x.to(dev), *d, bias.to(dev))
+    assert y.dtype == torch.bfloat16 and _rel(y.float().cpu().numpy(), ref) <= 2.0 ** -7      # float32 inside, bf16 out
+    monkeypatch.setattr(ops, "PREFILL", "nope")
+    with pytest.raises(RuntimeError, match="HTR_PREFILL"):
+        ops.linear(x.to(dev), *d)
+    monkeypatch.setattr(ops, "PREFILL", "w")
+    y_one = ops.linear_f32out(x[:24].to(dev), *d).cpu().numpy()
+    monkeypatch.setattr(ops, "LAUNCH_MAX_M", 8)                   # three launches of 8 rows, as the reference would
+    y_cut = ops.linear_f32out(x[:24].to(dev), *d).cpu().numpy()
+    r24 = _ref(oracle, qw, sc, su, sv, x[:24])
+    assert _rel(y_one, r24) <= REL_TOL and _rel(y_cut, r24) <= REL_TOL
+
+
 @pytest.mark.parametrize("K", [2, 3, 4, 5])
 @pytest.mark.parametrize("M", [1, 2, 3, 4, 8])
 @pytest.mark.parametrize("shape", [(256, 384), (1024, 4096), (4096, 1024)])

@@ -105,7 +105,8 @@ def test_apply_routes_to_ops_linear_and_counts(monkeypatch, tmp_path):
         return torch.zeros(*x.shape[:-1], 128, dtype=x.dtype)
     monkeypatch.setattr(ops, "linear", fake_linear)
     monkeypatch.setattr(vp, "_COUNT_FILE", str(tmp_path / "census"))
-    vp._COUNTS.clear()
+    vp._CENSUS.counts.clear()
+    vp._CENSUS.calls = 0
     x = torch.zeros(3, 128, dtype=torch.bfloat16)
     b = torch.zeros(128, dtype=torch.bfloat16)
     for _ in range(512):

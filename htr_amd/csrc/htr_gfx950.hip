@@ -296,9 +296,11 @@ struct LinearTail {
   unsigned long long group_part_stride;     // floats
 };
 
-constexpr int ROT_PAIRS = 32;  // (activation row, 128-column block) pairs a workgroup may rotate by itself: four per wave
+constexpr int ROT_PAIRS = 32;      // (activation row, 128-column block) pairs a workgroup rotates in one pass: four per wave
+constexpr int MAX_ROT_PASSES = 4;  // passes of the kernel variant for up to 8 rows over long chunks
+constexpr int MAX_ROT_PAIRS = ROT_PAIRS * MAX_ROT_PASSES;
 
-// LDS layout (dynamic): [xt: (M + 1) rows x row_halves f16][xs: M * nbl * 2 f32 (per tile parity)][sc: M f32][bs: 32 f32, scale per pair]
+// LDS layout (dynamic): [xt: (M + 1) rows x row_halves f16][xs: M * nbl * 2 f32 (per tile parity)][sc: M f32][bs: 128 f32, scale per pair]
 //                       [fin: segfin x M x 128 f32, partials of the row blocks this workgroup finishes]
 // nbl = number of distinct column blocks a chunk touches = min(chunk, n / 128)
 // One rotated 128-column block is stored as [columns 0..7 of tiles 0..7][columns 8..15 of tiles 0..7] (2 x 64 halves), and
@@ -307,7 +309,7 @@ constexpr int ROT_PAIRS = 32;  // (activation row, 128-column block) pairs a wor
 __host__ __device__ inline int xt_row_halves(int nbl) { return nbl * 128 + 16; }
 __device__ __forceinline__ int xt_slot(int j) { return ((j >> 3) & 1) * 64 + (j >> 4) * 8 + (j & 7); }   // element j of a block
 __host__ __device__ inline size_t lds_fin_offset(int M, int nbl) {
-  return ((size_t)(M + 1) * xt_row_halves(nbl) * 2 + (size_t)M * nbl * 4 * 2 + (size_t)M * 4 + ROT_PAIRS * 4 + 15) / 16 * 16;
+  return ((size_t)(M + 1) * xt_row_halves(nbl) * 2 + (size_t)M * nbl * 4 * 2 + (size_t)M * 4 + MAX_ROT_PAIRS * 4 + 15) / 16 * 16;
 }
 __host__ __device__ inline size_t lds_bytes(int M, int nbl, int segfin) {
   return lds_fin_offset(M, nbl) + (size_t)segfin * M * 128 * 4;
@@ -330,6 +332,46 @@ __device__ __forceinline__ int block_scale_exponent(uint32_t amax_bits) {
   const int l2 = ex - 127;
   if (l2 >= -8 && l2 <= 14) return 0;
   return max(-100, l2 - 13);
+}
+
+// ---- rotation of four 128-element blocks on the matrix unit: H128 = H4 (x) H32 over the element index i = 32 a + c, so
+// a block is a 4 x 32 matrix X and H128 x = H4 . X . H32 (unnormalised).  The four blocks of a wave are the 16 rows
+// (block p, a) of one MFMA A operand: lane (k-group gk = lane / 16, row = lane % 16 = 4 p + a) brings the 8
+// consecutive 16-bit elements 32 a + 8 gk .. + 7 of block p (xr) and the su byte that holds their signs (sb).  The
+// products are exact (operands are the activations themselves and +-1), accumulated in float32.  Result: lane
+// (p = lane / 16, j = lane % 16) holds y[h][a'] = element 32 a' + 16 h + j of block p.
+__device__ __forceinline__ void rotate4_mfma(const u4& xr, uint32_t sb, bool is_bf16, int lane, float (&y)[2][4]) {
+  uint32_t xs4[4] = {xr.x, xr.y, xr.z, xr.w};
+#pragma unroll
+  for (int d = 0; d < 4; ++d)                                    // elements 2d (low half), 2d + 1 (high half): su bits 2d, 2d + 1
+    xs4[d] ^= ((sb << (15 - 2 * d)) & 0x8000u) | ((sb << (30 - 2 * d)) & 0x80000000u);
+  // B operand: H32[k][c'] = (-1)^popcount(k & c') for k = 8 gk + i (dword d holds i = 2d, 2d + 1) and
+  // c' = 16 h + j, j = lane % 16; as 16-bit ones with the sign bit set where the parity is odd
+  const int j = lane & 15, gk = lane >> 4;
+  const uint32_t one2 = is_bf16 ? 0x3F803F80u : 0x3C003C00u;
+  const uint32_t o1 = (j & 1) ? 0x80000000u : 0u;
+  const uint32_t e1 = (j & 2) ? 0x80008000u : 0u;
+  const uint32_t e2 = (j & 4) ? 0x80008000u : 0u;
+  const uint32_t f3 = ((gk & 1) && (j & 8)) ? 0x80008000u : 0u;   // k bit 3 with c' bit 3
+  const uint32_t f4m = (gk & 2) ? 0x80008000u : 0u;               // k bit 4 with c' bit 4 (h = 1)
+  const uint32_t b0 = one2 ^ o1 ^ f3;
+  const u4 hb0 = {b0, b0 ^ e1, b0 ^ e2, b0 ^ e1 ^ e2};
+  const u4 hb1 = {hb0.x ^ f4m, hb0.y ^ f4m, hb0.z ^ f4m, hb0.w ^ f4m};
+  const u4 xa = {xs4[0], xs4[1], xs4[2], xs4[3]};
+  const f4 zero4 = {0.f, 0.f, 0.f, 0.f};
+  f4 t0, t1;
+  if (is_bf16) {
+    t0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(b8, xa), __builtin_bit_cast(b8, hb0), zero4, 0, 0, 0);
+    t1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(b8, xa), __builtin_bit_cast(b8, hb1), zero4, 0, 0, 0);
+  } else {
+    t0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, xa), __builtin_bit_cast(h8, hb0), zero4, 0, 0, 0);
+    t1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, xa), __builtin_bit_cast(h8, hb1), zero4, 0, 0, 0);
+  }
+  // D: lane (p = lane / 16, j), register a: T[p][a][16 h + j].  H4 over a gives element 32 a' + 16 h + j.
+  const float u0 = t0.x + t0.y, u1 = t0.x - t0.y, u2 = t0.z + t0.w, u3 = t0.z - t0.w;
+  y[0][0] = u0 + u2; y[0][1] = u1 + u3; y[0][2] = u0 - u2; y[0][3] = u1 - u3;
+  const float w0 = t1.x + t1.y, w1 = t1.x - t1.y, w2 = t1.z + t1.w, w3 = t1.z - t1.w;
+  y[1][0] = w0 + w2; y[1][1] = w1 + w3; y[1][2] = w0 - w2; y[1][3] = w1 - w3;
 }
 
 // Rotation of all activation rows ahead of the linear kernel (used where every workgroup rotating its own column
@@ -482,7 +524,7 @@ __device__ __forceinline__ uint32_t load_status(const uint32_t* status) {
 constexpr int FLAG_LANES = 1 << 4;     // kernel flag: chunk ids are dealt to the XCDs in eight lanes (see k_linear)
 constexpr int FLAG_LANE_LEN_SHIFT = 8; // with FLAG_LANES: grid / 8 in the bits from here up (no read of the hidden grid-size argument)
 
-template <int K, int MB, int P, int D, bool PREROT>
+template <int K, int MB, int P, int D, bool PREROT, int RP>
 __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restrict__ qw_a, const void* __restrict__ x_a,
                                                        const uint8_t* __restrict__ su_a, float* __restrict__ part_a,
                                                        int m, int n, int M_a, int chunk, int flags,
@@ -550,8 +592,9 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
   // (k-group gk = lane / 16, row = lane % 16 = 4 p + a) loads the 8 consecutive elements 32 a + 8 gk .. + 7 of its pair
   // (16 bytes) and the one su byte that holds their signs.  Descriptors over x and su: a pair beyond the chunk's last
   // one gets an out-of-range offset and reads zeros, so the loads issue back to back without branches.
-  u4 xr = {0u, 0u, 0u, 0u};
-  uint32_t sb = 0u;
+  // RP passes of 32 pairs (template: 1, or MAX_ROT_PASSES for many rows over long chunks); all loads go out up front.
+  u4 xr[RP];
+  uint32_t sb[RP];
   constexpr int COPY_REGS = 4;
   u4 cp[COPY_REGS];
   int cdst[COPY_REGS];
@@ -562,15 +605,23 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
     constexpr int OUT_OF_RANGE = 0x7FFFFF00;
     // every offset first, then the loads back to back: with address arithmetic (and its branches) between two loads
     // the compiler waits for the first load to return before it issues the second one and the weight stream behind it
-    const int pi = 4 * w + ((lane & 15) >> 2), a = lane & 3, gk = lane >> 4;
-    const bool live = pi < npairs;
-    const int prow = row_of_pair(pi), pli = pi - prow * nbl;
-    const int col = pair_col(pli) + 32 * a + 8 * gk;
-    const int xoff = live ? (prow * n + col) * 2 : OUT_OF_RANGE;
-    const int soff = live ? col >> 3 : OUT_OF_RANGE;
+    const int a = lane & 3, gk = lane >> 4;
+    int xoff[RP], soff[RP];
+#pragma unroll
+    for (int r = 0; r < RP; ++r) {
+      const int pi = ROT_PAIRS * r + 4 * w + ((lane & 15) >> 2);
+      const bool live = pi < npairs;
+      const int prow = row_of_pair(pi), pli = pi - prow * nbl;
+      const int col = pair_col(pli) + 32 * a + 8 * gk;
+      xoff[r] = live ? (prow * n + col) * 2 : OUT_OF_RANGE;
+      soff[r] = live ? col >> 3 : OUT_OF_RANGE;
+    }
     HTR_PIN();
-    xr = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xoff, 0, 0);
-    sb = (uint32_t)(uint8_t)__builtin_amdgcn_raw_buffer_load_b8(srsrc, soff, 0, 0);
+#pragma unroll
+    for (int r = 0; r < RP; ++r) {
+      xr[r] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, xoff[r], 0, 0);
+      sb[r] = (uint32_t)(uint8_t)__builtin_amdgcn_raw_buffer_load_b8(srsrc, soff[r], 0, 0);
+    }
     HTR_PIN();
   } else {
     // with pre-rotated activations: 16-byte pieces of this chunk's x~ slice, through a descriptor over x~ so that the
@@ -660,42 +711,12 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
   // block of the chunk has another scale, the products are scaled per block (see consume()).  No exchange between
   // waves, so one barrier between the rotation and the first product.
   if constexpr (!PREROT) {
-    if (4 * w < npairs) {                                            // uniform
-      const bool is_bf16 = x_dtype == HTR_BF16;
-      uint32_t xs4[4] = {xr.x, xr.y, xr.z, xr.w};
 #pragma unroll
-      for (int d = 0; d < 4; ++d)                                    // elements 2d (low half), 2d + 1 (high half): su bits 2d, 2d + 1
-        xs4[d] ^= ((sb << (15 - 2 * d)) & 0x8000u) | ((sb << (30 - 2 * d)) & 0x80000000u);
-      // B operand: H32[k][c'] = (-1)^popcount(k & c') for k = 8 gk + i (dword d holds i = 2d, 2d + 1) and
-      // c' = 16 h + j, j = lane % 16; as 16-bit ones with the sign bit set where the parity is odd
-      const int j = lane & 15, gk = lane >> 4;
-      const uint32_t one2 = is_bf16 ? 0x3F803F80u : 0x3C003C00u;
-      const uint32_t o1 = (j & 1) ? 0x80000000u : 0u;
-      const uint32_t e1 = (j & 2) ? 0x80008000u : 0u;
-      const uint32_t e2 = (j & 4) ? 0x80008000u : 0u;
-      const uint32_t f3 = ((gk & 1) && (j & 8)) ? 0x80008000u : 0u;   // k bit 3 with c' bit 3
-      const uint32_t f4m = (gk & 2) ? 0x80008000u : 0u;               // k bit 4 with c' bit 4 (h = 1)
-      const uint32_t b0 = one2 ^ o1 ^ f3;
-      const u4 hb0 = {b0, b0 ^ e1, b0 ^ e2, b0 ^ e1 ^ e2};
-      const u4 hb1 = {hb0.x ^ f4m, hb0.y ^ f4m, hb0.z ^ f4m, hb0.w ^ f4m};
-      const u4 xa = {xs4[0], xs4[1], xs4[2], xs4[3]};
-      const f4 zero4 = {0.f, 0.f, 0.f, 0.f};
-      f4 t0, t1;
-      if (is_bf16) {
-        t0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(b8, xa), __builtin_bit_cast(b8, hb0), zero4, 0, 0, 0);
-        t1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(b8, xa), __builtin_bit_cast(b8, hb1), zero4, 0, 0, 0);
-      } else {
-        t0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, xa), __builtin_bit_cast(h8, hb0), zero4, 0, 0, 0);
-        t1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h8, xa), __builtin_bit_cast(h8, hb1), zero4, 0, 0, 0);
-      }
-      // D: lane (p = lane / 16, j), register a: T[p][a][16 h + j].  H4 over a gives element 32 a' + 16 h + j.
+    for (int r = 0; r < RP; ++r) {
+    if (ROT_PAIRS * r + 4 * w < npairs) {                            // uniform
+      const int j = lane & 15;
       float y[2][4];
-      {
-        const float u0 = t0.x + t0.y, u1 = t0.x - t0.y, u2 = t0.z + t0.w, u3 = t0.z - t0.w;
-        y[0][0] = u0 + u2; y[0][1] = u1 + u3; y[0][2] = u0 - u2; y[0][3] = u1 - u3;
-        const float w0 = t1.x + t1.y, w1 = t1.x - t1.y, w2 = t1.z + t1.w, w3 = t1.z - t1.w;
-        y[1][0] = w0 + w2; y[1][1] = w1 + w3; y[1][2] = w0 - w2; y[1][3] = w1 - w3;
-      }
+      rotate4_mfma(xr[r], sb[r], x_dtype == HTR_BF16, lane, y);
       // largest |value| of the pair: 8 in the lane, then over the 16 lanes of the row
       float mx = fmaxf(fmaxf(fmaxf(fabsf(y[0][0]), fabsf(y[0][1])), fmaxf(fabsf(y[0][2]), fabsf(y[0][3]))),
                        fmaxf(fmaxf(fabsf(y[1][0]), fabsf(y[1][1])), fmaxf(fabsf(y[1][2]), fabsf(y[1][3]))));
@@ -704,7 +725,7 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
       mu = max(mu, dpp_mov_u32<0x141>(mu)); mu = max(mu, dpp_mov_u32<0x140>(mu));
       const int e = block_scale_exponent(mu);
       const float f = pow2f(-e) * INV_SQRT128;
-      const int po = 4 * w + (lane >> 4);
+      const int po = ROT_PAIRS * r + 4 * w + (lane >> 4);
       const bool live_o = po < npairs;
       const int prow_o = row_of_pair(po), pli_o = po - prow_o * nbl;
       _Float16* dst = xt + (size_t)prow_o * rowh + pli_o * 128 + (j >> 3) * 64 + (j & 7);
@@ -725,6 +746,7 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
         s_xs[2 * po] = sums[0]; s_xs[2 * po + 1] = sums[1];
         s_bs[po] = pow2f(e);
       }
+    }
     }
   }
 
@@ -792,7 +814,12 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
   // does any block this workgroup rotated carry a scale other than 1?  (uniform; never with pre-rotated activations,
   // whose scale is one per row)
   bool scaled = false;
-  if constexpr (!PREROT) scaled = __any(s_bs[min(lane, npairs - 1)] != 1.f) != 0;
+  if constexpr (!PREROT) {
+    bool other = false;
+#pragma unroll
+    for (int r = 0; r < (RP * ROT_PAIRS + 63) / 64; ++r) other |= s_bs[min(lane + 64 * r, npairs - 1)] != 1.f;
+    scaled = __any(other) != 0;
+  }
 
   f4 acc[MB][2];
 #pragma unroll
@@ -1751,9 +1778,10 @@ inline bool plan_for_chunk(int m, int n, int M, int chunk, Plan& pl) {
   pl.nbl = chunk < nblk ? chunk : nblk;
   pl.lds = lds_bytes(M, pl.nbl, pl.segfin);
   if (pl.lds > (size_t)LDS_BUDGET) return false;
-  // a workgroup rotates its own column blocks while that is at most ROT_PAIRS (row, block) pairs; beyond that the
-  // activations are rotated once, ahead of the launch
-  pl.prerot = M * pl.nbl > ROT_PAIRS ? 1 : 0;
+  // a workgroup rotates its own column blocks while that is at most ROT_PAIRS (row, block) pairs (MAX_ROT_PAIRS with up
+  // to eight rows: the kernel variant with several passes); beyond that the activations are rotated once, ahead of
+  // the launch
+  pl.prerot = M * pl.nbl > (M <= 8 ? MAX_ROT_PAIRS : ROT_PAIRS) ? 1 : 0;
   return true;
 }
 
@@ -1796,7 +1824,8 @@ inline bool search_plan(int m, int n, int M, int nsplit, Plan& pl) {
                                     : fill2 * (rows * 0.55 * steps + 0.5 + 0.1 * M);
     // hand-over: the contributors' slots are read eight per round trip to memory (0.45 us each)
     const double handover = 0.45 * ((contributors - 1 + 7) / 8);
-    const double t = 4.5 + handover + (c.prerot ? 3.0 + 0.1 * M : 0.0) + body;
+    const int passes = (M * c.nbl + ROT_PAIRS - 1) / ROT_PAIRS;      // rotation passes inside the kernel, 0.3 us each after the first
+    const double t = 4.5 + handover + (c.prerot ? 3.0 + 0.1 * M : 0.3 * (passes - 1)) + body;
     if (t < best) { best = t; pl = c; found = true; }
   }
   return found;
@@ -1875,12 +1904,12 @@ struct LinearLaunch {
   LinearTail tail;
 };
 
-template <int K, int MB, bool DEEP, bool PREROT> int launch_linear_v(const LinearLaunch& a, int grid, size_t lds, hipStream_t st) {
+template <int K, int MB, bool DEEP, bool PREROT, int RP = 1> int launch_linear_v(const LinearLaunch& a, int grid, size_t lds, hipStream_t st) {
   constexpr int P = K <= 4 ? 4 : (K <= 6 ? 3 : 2);          // wave-steps of weights in flight
   constexpr int D = DEEP && P >= 4 ? 4 : 2;                 // steps decoded ahead of the activation exchange
   lds = balanced_lds_request(lds, grid * a.problems);
-  HTR_CHECK_HIP((allow_full_lds<k_linear<K, MB, P, D, PREROT>>()));
-  HTR_CHECK_HIP(launch_kernel(k_linear<K, MB, P, D, PREROT>, dim3(grid, a.problems), dim3(WG_THREADS), lds, st, a.qw, a.x, a.su, a.part,
+  HTR_CHECK_HIP((allow_full_lds<k_linear<K, MB, P, D, PREROT, RP>>()));
+  HTR_CHECK_HIP(launch_kernel(k_linear<K, MB, P, D, PREROT, RP>, dim3(grid, a.problems), dim3(WG_THREADS), lds, st, a.qw, a.x, a.su, a.part,
                               a.m, a.n, a.M, a.chunk, a.flags, a.nblk_magic, a.tail));
   return HTR_OK;
 }
@@ -1888,6 +1917,10 @@ template <int K, int MB, bool DEEP, bool PREROT> int launch_linear_v(const Linea
 // block and chunks whose prologue latency is a large part of the kernel); long chunks prefer occupancy.
 template <int K, bool PREROT> int launch_linear_kr(const LinearLaunch& a, int mb, int grid, size_t lds, hipStream_t st) {
   const bool deep = a.chunk <= 8;
+  if constexpr (!PREROT) {                 // more pairs than one pass rotates: the variant with several passes (up to 8 rows)
+    const int nblk = a.n / 128;
+    if (mb == 1 && a.M * (a.chunk < nblk ? a.chunk : nblk) > ROT_PAIRS) return launch_linear_v<K, 1, false, false, MAX_ROT_PASSES>(a, grid, lds, st);
+  }
   switch (mb) {
     case 1: return deep ? launch_linear_v<K, 1, true, PREROT>(a, grid, lds, st) : launch_linear_v<K, 1, false, PREROT>(a, grid, lds, st);
     case 2: return launch_linear_v<K, 2, false, PREROT>(a, grid, lds, st);

@@ -210,6 +210,38 @@ def test_large_activations_do_not_overflow(dev, oracle):
         assert _rel(y[r], ref[r]) <= REL_TOL
 
 
+@pytest.mark.parametrize("M,chunk", [(8, 16), (5, 11), (3, 32), (8, 9), (2, 20)])
+def test_workgroups_rotate_many_blocks_themselves(dev, oracle, M, chunk, monkeypatch):
+    """Up to 8 rows over long chunks: more than 32 and at most 128 (row, block) pairs per workgroup are rotated inside the
+    kernel in several passes, no separate rotation launch.  Rows of very different magnitude (a huge one, a tiny one, a
+    zero one, one whose blocks differ by 2^30) take the per-block scales of every pass."""
+    import ctypes
+    from htr_amd import _native, ops
+    print(f"in-kernel rotation, several passes M={M} chunk={chunk}", flush=True)
+    m, n = 1024, 4096
+    out = (ctypes.c_int * 6)()
+    assert _native.lib().htr_linear_plan(m, n, 4, M, chunk, out) == 0
+    assert out[4] == 0 and 32 < M * out[3] <= 128                       # not pre-rotated, more than one pass
+    qw, sc, su, sv, x = _case(m, n, 4, M, 3100 + M, torch.bfloat16)
+    x = x.float()
+    x[0] *= 2.0 ** 20
+    x[1] *= 2.0 ** -22
+    if M > 2:
+        x[2] = 0.0
+    if M > 3:
+        x[3, 1024:2048] *= 2.0 ** 30
+    x = x.bfloat16()
+    monkeypatch.setattr(ops, "NSPLIT", chunk)
+    y = ops.linear_f32out(x.to(dev), *[t.to(dev) for t in (qw, sc, su, sv)]).cpu().numpy()
+    ref = _ref(oracle, qw, sc, su, sv, x)
+    assert np.all(np.isfinite(y))
+    for r in range(M):
+        if r == 2:
+            assert not np.any(y[r])
+        else:
+            assert _rel(y[r], ref[r]) <= REL_TOL, (r, _rel(y[r], ref[r]))
+
+
 @pytest.mark.parametrize("M", [1, 3, 9])
 def test_zero_tiny_and_non_finite_activations(dev, oracle, M):
     """All-zero rows give exactly the bias, rows of 1e-30 keep their relative accuracy, and an infinity or a NaN in a

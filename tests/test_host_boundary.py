@@ -91,7 +91,7 @@ def test_launch_plan_is_consistent(L, m, n, M):
     assert chunk >= 1 and (wgs - 1) * chunk < rbs * nblk <= wgs * chunk          # chunks tile the step space exactly
     assert nbl == min(chunk, nblk) and lds <= 64 * 1024
     assert segfin == (chunk + nblk - 1) // nblk                                  # row blocks that can end inside one chunk
-    assert prerot == (1 if M * nbl > 32 else 0)                                  # a workgroup rotates at most 32 pairs itself
+    assert prerot == (1 if M * nbl > (128 if M <= 8 else 32) else 0)                                  # a workgroup rotates at most 32 pairs itself
     # an explicit chunk length is honoured
     assert L.htr_linear_plan(m, n, 4, M, 1, out) == 0
     if out[0] == 1:

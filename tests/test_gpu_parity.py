@@ -491,3 +491,55 @@ def test_seeded_sweep_of_shapes_rows_and_widths(dev, oracle, monkeypatch):
         worst = max(worst, err)
         assert err <= REL_TOL, (case, m, n, K, M, dtype, with_bias, err)
     print(f"sweep worst relative error {worst:.2e}", flush=True)
+
+
+def test_seeded_random_cases_through_the_c_abi(dev, oracle):
+    """120 seeded random problems straight through htr_linear: K 2..8, m up to 2048, n up to 3072, 1..40 rows, library
+    plans and explicit chunk lengths, bf16 / f16 activations, all three output types, bias or none, a zero row, a block
+    2^14 times larger than its neighbours, tiny and huge magnitudes.  Every case runs twice on one workspace, which must
+    come back clean (status word and partial slots zero)."""
+    import random
+    from htr_amd import _native, wire
+    L = _native.lib()
+    rng = random.Random(20261125)
+    ydts = {0: torch.bfloat16, 1: torch.float16, 2: torch.float32}
+    tols = {0: 2.0 ** -8 + REL_TOL, 1: 2.0 ** -11 + REL_TOL, 2: REL_TOL}
+    for it in range(120):
+        K = rng.choice([2, 3, 4, 4, 4, 5, 6, 7, 8])
+        m, n = 128 * rng.randint(1, 16), 128 * rng.randint(1, 24)
+        M = rng.choice([1, 1, 2, 3, 4, 5, 6, 7, 8, 8, 9, 12, 16, 17, 31, 40])
+        nsplit = rng.randint(1, min((m // 128) * (n // 128), 40)) if M <= 8 and rng.random() < 0.6 else 0
+        dt, ydt = rng.choice([torch.bfloat16, torch.float16]), rng.choice([0, 1, 2])
+        scale = rng.choice([1.0, 1e-3]) if dt == torch.float16 or ydt == 1 else rng.choice([1.0, 1.0, 3e4, 1e-6])   # inside f16's range
+        print(f"random case {it}: K{K} {m}x{n} M{M} nsplit {nsplit} {dt} y{ydt} x{scale}", flush=True)
+        need = L.htr_workspace_bytes(m, n, K, M, nsplit)
+        if need == 0:
+            continue                                                    # no plan for this explicit chunk length
+        qw, sc, su, sv = wire.synth_linear(m, n, K, 1000 + it)
+        x = (wire.synth_activation(M, n, 2000 + it, torch.float32) * scale).to(dt)
+        if M > 2 and rng.random() < 0.5:
+            x[1] = 0
+        if rng.random() < 0.3 and dt == torch.bfloat16 and ydt != 1:
+            x[0, :128] *= 2.0 ** 14
+        d = [t.to(dev) for t in (qw, sc, su, sv)]
+        xd = x.to(dev)
+        y = torch.empty(M, m, dtype=ydts[ydt], device=dev)
+        bias = torch.randn(m, generator=torch.Generator().manual_seed(it)).to(ydts[ydt]).to(dev) if rng.random() < 0.5 else None
+        ws = torch.zeros(need, dtype=torch.uint8, device=dev)
+        for _ in range(2):
+            _native.check(L.htr_linear(d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), d[3].data_ptr(), xd.data_ptr(),
+                                       None if bias is None else bias.data_ptr(), y.data_ptr(), m, n, K, M,
+                                       _native.BF16 if dt == torch.bfloat16 else _native.F16, ydt, nsplit, ws.data_ptr(), ws.numel(),
+                                       torch.cuda.current_stream().cuda_stream))
+            torch.cuda.synchronize()
+        assert int(ws[:4].view(torch.int32)[0]) == 0 and not bool(ws[256:ws.numel() // 2].any()), "workspace not clean"
+        ref = oracle.c_linear(x.float().numpy(), qw.numpy(), sc.numpy(), su.numpy(), sv.numpy(),
+                              None if bias is None else bias.float().cpu().numpy().astype(np.float64))
+        got = y.float().cpu().numpy()
+        assert np.all(np.isfinite(got)), it
+        for r in range(M):
+            den = np.abs(ref[r]).max()
+            if den == 0:
+                assert not np.any(got[r]), (it, r)
+            else:
+                assert np.abs(got[r] - ref[r]).max() <= tols[ydt] * den, (it, r, float(np.abs(got[r] - ref[r]).max() / den))

@@ -470,6 +470,76 @@ __global__ __launch_bounds__(WG_THREADS) void k_rotate(const void* __restrict__ 
   }
 }
 
+// The same for 16-bit activations whose rows start on 16-byte boundaries, on the matrix unit (rotate4_mfma): a wave
+// rotates four blocks, a workgroup 32 blocks of one activation row; grid = (blocks / 32 rounded up, rows).  About a
+// seventh of the vector instructions of the butterfly version per block, which shows where the rotation is not just
+// latency: 128 rows of 14336 columns take 8.6 us there.
+__global__ __launch_bounds__(WG_THREADS) void k_rotate_mfma(const void* __restrict__ x, const uint8_t* __restrict__ su, int n, int is_bf16,
+                                                            _Float16* __restrict__ xt_g, float* __restrict__ xs_g, float* __restrict__ sc_g) {
+  __shared__ uint32_t s_amax[WG_WAVES];
+  const int lane = threadIdx.x & 63, w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int mrow = blockIdx.y, nblk = n >> 7;
+  const int b0 = blockIdx.x * 4 * WG_WAVES + 4 * w;        // first of this wave's four blocks
+  const int gk = lane >> 4, j = lane & 15;
+  const unsigned char* xrow = (const unsigned char*)x + (size_t)mrow * n * 2;
+  const __amdgpu_buffer_rsrc_t rrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)xrow, 0, n * 2, 0x00020000);
+  const __amdgpu_buffer_rsrc_t srsrc = __builtin_amdgcn_make_buffer_rsrc((void*)su, 0, n >> 3, 0x00020000);
+  constexpr int OUT_OF_RANGE = 0x7FFFFF00;
+  // own elements first (lane (gk, row = 4 p + a) brings elements 32 a + 8 gk .. + 7 of block b0 + p), then the scan of
+  // the row for max|x|, all loads back to back; blocks beyond the row read zeros
+  const int col = (b0 + (j >> 2)) * 128 + 32 * (j & 3) + 8 * gk;
+  const bool live = b0 + (j >> 2) < nblk;
+  const u4 xr = __builtin_amdgcn_raw_buffer_load_b128(rrsrc, live ? col * 2 : OUT_OF_RANGE, 0, 0);
+  const uint32_t sb = (uint32_t)(uint8_t)__builtin_amdgcn_raw_buffer_load_b8(srsrc, live ? col >> 3 : OUT_OF_RANGE, 0, 0);
+  uint32_t m16 = 0u;                                       // max of the sign-cleared halves: |values| compare like their bits
+  for (int base = (int)threadIdx.x * 16; base < n * 2; base += 4 * WG_THREADS * 16) {
+    u4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) v[u] = __builtin_amdgcn_raw_buffer_load_b128(rrsrc, base + u * WG_THREADS * 16, 0, 0);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const uint32_t d[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+#pragma unroll
+      for (int k = 0; k < 4; ++k) m16 = max(m16, max(d[k] & 0x7FFFu, (d[k] >> 16) & 0x7FFFu));
+    }
+  }
+  m16 = wave_max_u32(m16);
+  if (lane == 0) s_amax[w] = m16;
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < WG_WAVES; ++k) m16 = max(m16, s_amax[k]);
+  float amax = is_bf16 ? bf16_bits_to_float((uint16_t)m16) : f16_bits_to_float((uint16_t)m16);
+  if (amax != amax) amax = __uint_as_float(0x7F800000u);   // a NaN anywhere: treat the row as unbounded (scale 1)
+  const int e = scale_exponent(amax);
+  const float f = pow2f(-e) * INV_SQRT128;
+  if (threadIdx.x == 0 && blockIdx.x == 0) sc_g[mrow] = pow2f(e);
+  if (b0 >= nblk) return;                                  // uniform per wave: none of its blocks exists
+  float y[2][4];
+  rotate4_mfma(xr, sb, is_bf16 != 0, lane, y);
+  const int b_o = b0 + gk;                                 // lane (p = lane / 16, j) holds elements 32 a' + 16 h + j of block b0 + p
+  const bool live_o = b_o < nblk;
+  HTR_GLOBAL _Float16* dst = (HTR_GLOBAL _Float16*)xt_g + (size_t)mrow * n + b_o * 128 + j;
+  float r[2][4];
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+      const _Float16 hv = (_Float16)(y[h][a] * f);
+      if (live_o) dst[32 * a + 16 * h] = hv;
+      r[h][a] = (float)hv;
+    }
+  // sums of the rounded values: even tiles (h = 0), odd tiles (h = 1), columns 0..63 (a < 2), columns 64..127
+  f4 sm = {(r[0][0] + r[0][1]) + (r[0][2] + r[0][3]), (r[1][0] + r[1][1]) + (r[1][2] + r[1][3]),
+           (r[0][0] + r[0][1]) + (r[1][0] + r[1][1]), (r[0][2] + r[0][3]) + (r[1][2] + r[1][3])};
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    float v = sm[c];
+    v += dpp_mov<0xB1>(v); v += dpp_mov<0x4E>(v); v += dpp_mov<0x141>(v); v += dpp_mov<0x140>(v);
+    sm[c] = v;
+  }
+  if (live_o && j == 0) *(HTR_GLOBAL f4*)((HTR_GLOBAL float*)xs_g + ((size_t)mrow * nblk + b_o) * 4) = sm;
+}
+
 template <int K> struct DecodedStep { h8 a[4]; };   // MFMA A operands of one step: (row 2q | 2q+1) x (columns 0..7 | 8..15)
 
 template <int K> __device__ __forceinline__ void decode_step(const StreamRegs<K>& r, int hist, DecodedStep<K>& d) {
@@ -1986,6 +2056,17 @@ inline bool wants_batch(int M, int nsplit, int m) {
   return M >= BATCH_MIN_M || (M >= 6 && m / 128 >= 192);
 }
 
+// Rotation of all rows of x ahead of a linear launch: on the matrix unit for 16-bit rows on 16-byte boundaries, else the
+// butterfly kernel (float32, odd alignments)
+inline hipError_t launch_rotation(const void* x, const uint8_t* su, int n, int M, int x_dtype, const LinearTail& t, hipStream_t st) {
+  static const bool mfma_on = getenv("HTR_ROTATE_MFMA") == nullptr || atoi(getenv("HTR_ROTATE_MFMA")) != 0;
+  if (mfma_on && x_dtype != HTR_F32 && ((uintptr_t)x & 15) == 0)
+    return launch_kernel(k_rotate_mfma, dim3((n / 128 + 4 * WG_WAVES - 1) / (4 * WG_WAVES), M), dim3(WG_THREADS), 0, st, x, su, n,
+                         x_dtype == HTR_BF16 ? 1 : 0, (_Float16*)t.xt_g, (float*)t.xs_g, (float*)t.sc_g);
+  return launch_kernel(k_rotate, dim3((n / 128 + WG_WAVES - 1) / WG_WAVES, M), dim3(WG_THREADS), 0, st, x, su, n, x_dtype,
+                       (_Float16*)t.xt_g, (float*)t.xs_g, (float*)t.sc_g, (const htr_group_entry*)nullptr, 0ull);
+}
+
 #define HTR_FOR_K(K, EXPR)                 \
   switch (K) {                             \
     case 2: { constexpr int KK = 2; EXPR; } break; \
@@ -2105,8 +2186,7 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
     t.chunk_magic = 0;
     t.group = nullptr; t.group_prerot_stride = 0; t.group_part_stride = 0;
     hipStream_t st = (hipStream_t)stream;
-    HTR_CHECK_HIP(launch_kernel(k_rotate, dim3((n / 128 + WG_WAVES - 1) / WG_WAVES, M), dim3(WG_THREADS), 0, st, x, (const uint8_t*)su, n, x_dtype,
-                                (_Float16*)t.xt_g, (float*)t.xs_g, (float*)t.sc_g, (const htr_group_entry*)nullptr, 0ull));
+    HTR_CHECK_HIP(launch_rotation(x, (const uint8_t*)su, n, M, x_dtype, t, st));
     float* part = (float*)((unsigned char*)workspace + WS_HEADER);
     const int flags = x_dtype | (y_dtype << 2);
     HTR_FOR_K(K, return launch_batch_k<KK>((const uint32_t*)qweight, part, m, n, M, flags, t, bp, st));
@@ -2149,8 +2229,7 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
     t.xt_g = (const _Float16*)wsp;
     t.xs_g = (const float*)(wsp + align256((size_t)M * n * 2));
     t.sc_g = (const float*)(wsp + align256((size_t)M * n * 2) + align256((size_t)M * (n / 128) * 16));
-    HTR_CHECK_HIP(launch_kernel(k_rotate, dim3((n / 128 + WG_WAVES - 1) / WG_WAVES, M), dim3(WG_THREADS), 0, st, x, (const uint8_t*)su, n, x_dtype,
-                                (_Float16*)t.xt_g, (float*)t.xs_g, (float*)t.sc_g, (const htr_group_entry*)nullptr, 0ull));
+    HTR_CHECK_HIP(launch_rotation(x, (const uint8_t*)su, n, M, x_dtype, t, st));
   }
   HTR_FOR_K(K, return launch_linear_k<KK>(a, prerot, pl.mb, pl.wgs, pl.lds, st));
   return HTR_OK;

@@ -162,3 +162,13 @@ def test_product_never_imports_the_oracle():
                 if re.search(r"^\s*(from|import)\s+oracle\b", text, flags=re.M) or "libhtr_oracle" in text:
                     bad.append(f)
     assert bad == []
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The packed-linear path has no collectives: `bench.py --gpus N` with N above 1 says so and exits before it
+    touches a GPU."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 2 and "one GPU only" in r.stderr and r.stdout.strip() == ""

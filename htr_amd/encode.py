@@ -4,8 +4,8 @@ Same algorithm and call surface as htr/encode.py of the reference (encode_group,
 hook, htr/encode.py:1-110): rotate W and the Hessian with the randomized Hadamard transform, factor the damped
 Hessian, walk the 16-column blocks from the last to the first, search each block's 256-weight tiles with the trellis
 Viterbi, and feed the quantization error of a block forward into the columns not yet encoded.  The search runs in
-libhtr_gfx950.so (htr_viterbi, one workgroup per tile) when the tensors are on the GPU; the linear algebra around it is
-torch.  Results are HTR-W1 tensors plus the reconstruction `What`.
+libhtr_gfx950.so (htr_viterbi, one workgroup per tile) when the tensors are on the GPU (a torch version of the same
+formulation serves CPU tensors); the linear algebra around it is torch.  Results are HTR-W1 tensors plus the reconstruction `What`.
 """
 import torch
 
@@ -25,11 +25,10 @@ def viterbi(x, w, cb=None, K=4, tailbite=True):
     x, w: float32 [B, T <= 256] on a ROCm device.  cb is accepted for signature compatibility and must be the HTR
     codebook (the kernel evaluates it procedurally; another table is refused).  Returns int64 states [B, T].
     Costs that are NaN never win a comparison in the kernel, where torch.argmin in the reference returns the first NaN:
-    inputs with NaN give different (meaningless either way) states.
+    inputs with NaN give different (meaningless either way) states.  CPU tensors take viterbi_cpu.
     """
     if not x.is_cuda:
-        raise RuntimeError("htr_amd.encode.viterbi runs on a ROCm device only; for CPU tensors set encode.VITERBI to a "
-                           "CPU search with the signature (x, w, cb, K) -> states")
+        return viterbi_cpu(x, w, K, tailbite)                       # the reference falls back to its torch search too
     if cb is not None and cb.data_ptr() not in _CHECKED_CB:
         if cb.numel() != wire.S or not torch.equal(cb.detach().float().cpu().reshape(-1), wire.codebook_f32("cpu")):
             raise RuntimeError("viterbi: cb is not the HTR-W1 codebook; the GPU search evaluates that codebook only")
@@ -61,6 +60,51 @@ def viterbi(x, w, cb=None, K=4, tailbite=True):
             _native.check(L.htr_viterbi(x[b0:].data_ptr(), w[b0:].data_ptr(), nb, T, K, 1 if tailbite else 0,
                                         out[b0:].data_ptr(), ws.data_ptr(), ws.numel(), stream.cuda_stream))
     return out.long() & 0xFFFF
+
+
+def viterbi_cpu(x, w, K=4, tailbite=True):
+    """The same search with torch on the CPU, for tensors that are not on a GPU (the reference's fallback is its
+    portable search, htr/reference.py:6-50; this is the formulation of the GPU kernel instead).  Per step only the
+    minima over the 2^K predecessors are kept: M_t[low] = min_j cost_{t-1}[j Sj + low] with Sj = 65536 >> K, and
+    cost_t[s] = M_t[s >> K] + w_t (x_t - cb[s])^2; arithmetic float32 and unfused, first index among equal values, two
+    passes for tail-biting (free start, then start and end tied to the first pass's final low bits)."""
+    x = x.float().contiguous()
+    w = w.float().contiguous()
+    B, T = x.shape
+    if w.shape != x.shape or not 1 <= T <= 256 or not 2 <= K <= 8:
+        raise RuntimeError("viterbi wants x and w of one shape [B, T <= 256] and K in 2..8")
+    S, NB, SJ = wire.S, 1 << K, wire.S >> K
+    cb = wire.codebook_f32("cpu")
+    pred = torch.arange(S) >> K                                   # M entry that state s continues
+    rows = torch.arange(B)
+    j0 = None
+    for constrained in ([False, True] if tailbite else [False]):
+        M = torch.zeros(B, SJ)
+        if constrained:
+            M = torch.full((B, SJ), float("inf"))
+            M[rows, j0] = 0.0
+        back = torch.empty(B, max(T - 1, 0), SJ, dtype=torch.uint8)
+        for t in range(T):
+            d = x[:, t:t + 1] - cb[None, :]
+            cost = M[:, pred] + w[:, t:t + 1] * (d * d)
+            if t == T - 1:
+                break
+            M, arg = cost.view(B, NB, SJ).min(dim=1)              # over the top K bits j of s = j Sj + low
+            back[:, t] = arg.to(torch.uint8)
+        if constrained:
+            cost = torch.where((torch.arange(S) & (SJ - 1))[None, :] == j0[:, None], cost, torch.full_like(cost, float("inf")))
+        cost = torch.where(torch.isnan(cost), torch.full_like(cost, float("inf")), cost)       # NaN never wins, as in the kernel
+        final = cost.argmin(dim=1)
+        final = torch.where(torch.isinf(cost[rows, final]), torch.zeros_like(final), final)
+        j0 = final & (SJ - 1)
+    states = torch.empty(B, T, dtype=torch.int64)
+    s_t = final
+    states[:, T - 1] = s_t
+    for t in range(T - 1, 0, -1):
+        low = s_t >> K
+        s_t = back[rows, t - 1, low].long() * SJ + low
+        states[:, t - 1] = s_t
+    return states
 
 
 def block_rotate(W, bs=wire.RHT_BLOCK):

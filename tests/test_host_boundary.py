@@ -172,3 +172,18 @@ def test_bench_refuses_more_than_one_gpu():
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
     assert r.returncode == 2 and "one GPU only" in r.stderr and r.stdout.strip() == ""
+
+
+def test_fake_tensors_and_make_fx_go_through_the_registered_op():
+    """Tracers other than dynamo (FakeTensorMode, make_fx) never reach a data pointer: ops.linear hands tensor
+    subclasses to the registered op htr::linear, whose fake implementation gives the shape (the reference always
+    dispatches the op, htr/ops.py:107-122)."""
+    from torch._subclasses.fake_tensor import FakeTensorMode
+    from torch.fx.experimental.proxy_tensor import make_fx
+    from htr_amd import ops, wire
+    w = wire.synth_linear(256, 384, 4, 1)
+    with FakeTensorMode() as mode:
+        y = ops.linear(torch.empty(3, 5, 384, dtype=torch.bfloat16), *[mode.from_tensor(t) for t in w])
+        assert tuple(y.shape) == (3, 5, 256) and y.dtype == torch.bfloat16
+    g = make_fx(lambda x, qw, sc, su, sv: ops.linear(x, qw, sc, su, sv), tracing_mode="fake")(torch.empty(2, 384, dtype=torch.bfloat16), *w)
+    assert any("htr.linear" in str(n.target) for n in g.graph.nodes)

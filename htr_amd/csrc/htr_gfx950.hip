@@ -1115,9 +1115,11 @@ constexpr int BATCH_FIN_STRIDE = 128 + 4;    // floats per activation row of the
 // rows x 4 groups of 8 output rows) hit 64 different banks with each of their 8 values
 __device__ __forceinline__ int batch_fin_pos(int r) { return (r & 7) * 16 + (r >> 3); }
 
-template <int K, int MG, int P>
-__global__ __launch_bounds__(WG_THREADS, MG <= 2 ? 4 : 2) void k_linear_batch(const uint32_t* __restrict__ qw, float* __restrict__ part,
+template <int K, int MG, int P, bool ROT>
+__global__ __launch_bounds__(WG_THREADS, MG <= 2 && !ROT ? 4 : 2) void k_linear_batch(const uint32_t* __restrict__ qw, float* __restrict__ part,
+                                                             const void* __restrict__ x, const uint8_t* __restrict__ su,
                                                              int m, int n, int M, int S, int flags, const LinearTail t) {
+  static_assert(!ROT || MG == 1, "the variant that rotates its own activations holds 16 rows");
   extern __shared__ __align__(16) unsigned char lds[];
   const int lane = threadIdx.x & 63;
   const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
@@ -1133,11 +1135,15 @@ __global__ __launch_bounds__(WG_THREADS, MG <= 2 ? 4 : 2) void k_linear_batch(co
   // [2 column halves][M][132] partial of the workgroup.  Rows M .. 16 MG - 1 are staged like the others (they read out of
   // range: zeros), so every group of 16 rows is addressed alike.  With more than 64 rows the partial does not fit
   // behind the blocks and takes their place once the last step is done.
+  // ROT (up to 16 rows, up to 16 column blocks per split): no rotation launch; the workgroup rotates the activations
+  // of its own column blocks at the start (wave w: rows 2w and 2w + 1, four blocks per pass on the matrix unit, one
+  // power-of-two scale per row from max|x| over the split's columns) and keeps all of them in LDS, [cb blocks][16 rows]
+  // [136 halves] + [cb][16][2] sums: no staging and no barrier inside the loop.
   constexpr int ROWH = BATCH_ROWH, ROWS = 16 * MG, BUFH = ROWS * ROWH;
   constexpr bool FIN_OVER_BLOCKS = MG > 4;
   _Float16* xt = (_Float16*)lds;
-  float* s_xs = (float*)(lds + (size_t)2 * BUFH * 2);
-  float* s_sc = s_xs + 4 * ROWS;
+  float* s_xs = (float*)(lds + (size_t)(ROT ? cb : 2) * BUFH * 2);
+  float* s_sc = s_xs + (ROT ? cb * 2 * ROWS : 4 * ROWS);
   float* s_fin = FIN_OVER_BLOCKS ? (float*)lds : s_sc + ROWS;
 
   // ---- activation staging in 16-byte pieces (8 halves): piece pi of the block is row pi / 16, columns 8 (pi % 16) .. + 7;
@@ -1179,9 +1185,34 @@ __global__ __launch_bounds__(WG_THREADS, MG <= 2 ? 4 : 2) void k_linear_batch(co
       if (has_piece) *(u4*)(xt + q * BUFH + piece_lds[i]) = xg[set][i];
     if (has_sum) s_xs[q * 2 * ROWS + tid] = xsg[set];
   };
-  if (tid < ROWS) s_sc[tid] = tid < M ? t.sc_g[tid] : 0.f;
-  stage_load(c_begin, 0);
-  if constexpr (DIST == 2) stage_load(c_begin + 1, 1);
+  // ROT: the raw activations of this wave's two rows, eight passes of four blocks, all loads back to back
+  constexpr int RPASS = ROT ? 8 : 1;
+  u4 rx[RPASS];
+  uint32_t rsb[RPASS];
+  if constexpr (ROT) {
+    const __amdgpu_buffer_rsrc_t rawsrc = __builtin_amdgcn_make_buffer_rsrc((void*)x, 0, M * n * 2, 0x00020000);
+    const __amdgpu_buffer_rsrc_t sgnsrc = __builtin_amdgcn_make_buffer_rsrc((void*)su, 0, n >> 3, 0x00020000);
+    int xo[RPASS], so[RPASS];
+#pragma unroll
+    for (int r = 0; r < RPASS; ++r) {
+      const int row = 2 * w + (r >> 2), bl = 4 * (r & 3) + ((lane & 15) >> 2);          // block within the split
+      const int col = (c_begin + bl) * 128 + 32 * (lane & 3) + 8 * (lane >> 4);
+      const bool live = row < M && bl < nsteps;
+      xo[r] = live ? (row * n + col) * 2 : OUT_OF_RANGE;
+      so[r] = live ? col >> 3 : OUT_OF_RANGE;
+    }
+    HTR_PIN();
+#pragma unroll
+    for (int r = 0; r < RPASS; ++r) {
+      rx[r] = __builtin_amdgcn_raw_buffer_load_b128(rawsrc, xo[r], 0, 0);
+      rsb[r] = (uint32_t)(uint8_t)__builtin_amdgcn_raw_buffer_load_b8(sgnsrc, so[r], 0, 0);
+    }
+    HTR_PIN();
+  } else {
+    if (tid < ROWS) s_sc[tid] = tid < M ? t.sc_g[tid] : 0.f;
+    stage_load(c_begin, 0);
+    if constexpr (DIST == 2) stage_load(c_begin + 1, 1);
+  }
 
   // row constants of the output side (scale, sign, bias of rows lane and lane + 64), requested ahead of the weight stream by
   // the workgroups that finish rows of the row block, so that they have long arrived when they are needed
@@ -1240,7 +1271,7 @@ __global__ __launch_bounds__(WG_THREADS, MG <= 2 ? 4 : 2) void k_linear_batch(co
   constexpr int NB = AHEAD ? MG : 4;               // B register sets
   h8 B0[NB], B1[NB];
   float xsv[NB];
-  auto fetch_b = [&](int bsel, int mg, int set) {
+  auto fetch_b = [&](int bsel, int mg, int set) {       // bsel: staging buffer (0 / 1), or with ROT the block within the split
     const _Float16* bp = b_lane + bsel * BUFH + mg * 16 * ROWH;
     B0[set] = *(const h8*)bp;
     B1[set] = *(const h8*)(bp + 64);
@@ -1284,12 +1315,81 @@ __global__ __launch_bounds__(WG_THREADS, MG <= 2 ? 4 : 2) void k_linear_batch(co
     }
   };
 
-  // step 0: its block goes to buffer 0, the next block to come is requested, the first weights are decoded meanwhile
   static_assert(P % 2 == 0, "the block parity of a step must be static in the unrolled loop");
   const int hist = history_lane_byteaddr(lane);
+  DecodedStep<K> cur;
+  if constexpr (ROT) {
+    // ---- rotation of this wave's two rows.  Row scale from the raw values: |H128 x| / sqrt(128) <= sqrt(128) max|x|.
+    const bool is_bf16 = (flags & 3) == HTR_BF16;
+    const int j = lane & 15, gk = lane >> 4;
+#pragma unroll
+    for (int rr = 0; rr < 2; ++rr) {
+      uint32_t m16 = 0u;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const uint32_t d[4] = {rx[4 * rr + q].x, rx[4 * rr + q].y, rx[4 * rr + q].z, rx[4 * rr + q].w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) m16 = max(m16, max(d[k] & 0x7FFFu, (d[k] >> 16) & 0x7FFFu));
+      }
+      m16 = wave_max_u32(m16);
+      float amax = is_bf16 ? bf16_bits_to_float((uint16_t)m16) : f16_bits_to_float((uint16_t)m16);
+      if (amax != amax) amax = __uint_as_float(0x7F800000u);      // a NaN anywhere: treat the row as unbounded (scale 1)
+      const int e = scale_exponent(amax);
+      const float f = pow2f(-e) * INV_SQRT128;
+      const int row = 2 * w + rr;
+      if (lane == 0) s_sc[row] = row < M ? pow2f(e) : 0.f;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        if (4 * q >= nsteps) continue;                             // uniform: none of the pass's blocks exists
+        float y[2][4];
+        rotate4_mfma(rx[4 * rr + q], rsb[4 * rr + q], is_bf16, lane, y);
+        const int bl = 4 * q + gk;                                 // lane (p = lane / 16, j) holds elements 32 a' + 16 h + j of block 4 q + p
+        const bool live_o = bl < nsteps;
+        _Float16* dst = xt + (size_t)(bl * ROWS + row) * ROWH + (j >> 3) * 64 + (j & 7);
+        float lo = 0.f, hi = 0.f;
+#pragma unroll
+        for (int h = 0; h < 2; ++h)
+#pragma unroll
+          for (int a = 0; a < 4; ++a) {
+            const _Float16 hv = (_Float16)(y[h][a] * f);
+            if (live_o) dst[(2 * a + h) * 8] = hv;
+            if (a < 2) lo += (float)hv; else hi += (float)hv;       // columns 0..63 | 64..127
+          }
+        lo += dpp_mov<0xB1>(lo); lo += dpp_mov<0x4E>(lo); lo += dpp_mov<0x141>(lo); lo += dpp_mov<0x140>(lo);
+        hi += dpp_mov<0xB1>(hi); hi += dpp_mov<0x4E>(hi); hi += dpp_mov<0x141>(hi); hi += dpp_mov<0x140>(hi);
+        if (live_o && j == 0) { s_xs[(bl * ROWS + row) * 2] = lo; s_xs[(bl * ROWS + row) * 2 + 1] = hi; }
+      }
+    }
+    decode_step<K>(buf[0], hist, cur);
+    prefetch(buf[0]);
+    __syncthreads();
+    load_b(0);
+    // the loop: multiply step v, read the operands of step v + 1, decode it; no barrier, every block is in LDS
+    int v = 0;
+    for (; v + P < nsteps; v += P) {
+#pragma unroll
+      for (int pp = 0; pp < P; ++pp) {
+        multiply(cur, 0);
+        load_b(v + pp + 1);
+        decode_step<K>(buf[(pp + 1) % P], hist, cur);
+        prefetch(buf[(pp + 1) % P]);
+      }
+    }
+#pragma unroll
+    for (int pp = 0; pp < P; ++pp) {
+      if (v + pp < nsteps) {
+        multiply(cur, 0);
+        if (v + pp + 1 < nsteps) {
+          load_b(v + pp + 1);
+          decode_step<K>(buf[(pp + 1) % P], hist, cur);
+          prefetch(buf[(pp + 1) % P]);
+        }
+      }
+    }
+  } else {
+  // step 0: its block goes to buffer 0, the next block to come is requested, the first weights are decoded meanwhile
   stage_store(0);
   stage_load(c_begin + DIST, 0);
-  DecodedStep<K> cur;
   decode_step<K>(buf[0], hist, cur);
   prefetch(buf[0]);
   __syncthreads();
@@ -1315,6 +1415,7 @@ __global__ __launch_bounds__(WG_THREADS, MG <= 2 ? 4 : 2) void k_linear_batch(co
     if (v + pp + 1 < nsteps) step_with_next(v + pp, (pp + 1) & 1, buf[(pp + 1) % P]);
     else if (v + pp < nsteps) multiply(cur, pp & 1);
   }
+  }   // staged path
 
   // ---- this wave's partial (offset removed, activation scale undone) goes to its column half's copy in LDS
   float scl[MG];
@@ -2002,7 +2103,9 @@ template <int K> int launch_linear_k(const LinearLaunch& a, bool prerot, int mb,
 }
 
 // ---- batched kernel: split S of the column blocks per row block
-struct BatchPlan { int S, cb, wgs, mb; size_t lds; };
+struct BatchPlan { int S, cb, wgs, mb, rot; size_t lds; };
+constexpr int BATCH_ROT_MAX_M = 16;      // rows and column blocks per split up to which a workgroup of the batched kernel
+constexpr int BATCH_ROT_MAX_CB = 16;     // rotates its own activations (256 pairs, eight passes per wave) instead of a rotation launch
 constexpr int BATCH_MIN_M = 9;      // rows from which the library policy takes the batched kernel on every shape
 inline int batch_groups(int M) { return M <= 16 ? 1 : (M <= 32 ? 2 : (M <= 64 ? 4 : 8)); }   // groups of 16 activation rows
 inline size_t batch_lds_bytes(int M) {
@@ -2015,6 +2118,7 @@ inline bool make_batch_plan(int m, int n, int M, int want_S, BatchPlan& bp) {
   if ((long)M * n * 2 >= (1L << 31)) return false;          // the kernels address the rotated activations with 32-bit byte offsets
   bp.mb = batch_groups(M);
   bp.lds = batch_lds_bytes(M);
+  bp.rot = 0;
   // Measured on MI355X (K4, 6..128 rows, 1024..28672 output rows): one workgroup per CU is the best fill; every further
   // split adds partial traffic that grows with the rows (14336x4096, 32 rows: 2 splits 19.9 us, 4 splits 24.5; 128
   // rows: 39 against 48).  So: the largest split that keeps the grid within the CU count, among the splits that leave
@@ -2029,31 +2133,46 @@ inline bool make_batch_plan(int m, int n, int M, int want_S, BatchPlan& bp) {
     if (want_S > 0 && S != want_S) continue;
     bp.S = S; bp.cb = cb; bp.wgs = rbs * S; found = true;
   }
+  // Up to 16 rows over at most 16 column blocks per split, one workgroup per CU: every workgroup rotates its own slice
+  // (measured on MI355X, K4, 16 rows: see the launch comment in htr_linear).  HTR_BATCH_ROT=0 switches it off.
+  static const bool rot_on = getenv("HTR_BATCH_ROT") == nullptr || atoi(getenv("HTR_BATCH_ROT")) != 0;
+  if (found && rot_on && M <= BATCH_ROT_MAX_M && bp.cb <= BATCH_ROT_MAX_CB && bp.wgs <= NUM_CU) {
+    bp.rot = 1;
+    bp.lds = (size_t)bp.cb * 16 * BATCH_ROWH * 2 + (size_t)bp.cb * 32 * 4 + 16 * 4 + (size_t)2 * M * BATCH_FIN_STRIDE * 4;
+  }
   return found;
 }
 
-template <int K, int MB> int launch_batch_v(const uint32_t* qw, float* part, int m, int n, int M, int flags, const LinearTail& t,
-                                            const BatchPlan& bp, hipStream_t st) {
+struct BatchArgs { const uint32_t* qw; float* part; const void* x; const uint8_t* su; int m, n, M, flags; };
+template <int K, int MB, bool ROT> int launch_batch_v(const BatchArgs& a, const LinearTail& t, const BatchPlan& bp, hipStream_t st) {
   const size_t lds = balanced_lds_request(bp.lds, bp.wgs);
-  HTR_CHECK_HIP((allow_full_lds<k_linear_batch<K, MB, 4>>()));
-  HTR_CHECK_HIP(launch_kernel(k_linear_batch<K, MB, 4>, dim3(bp.S, m / 128), dim3(WG_THREADS), lds, st, qw, part, m, n, M, bp.S, flags, t));
+  HTR_CHECK_HIP((allow_full_lds<k_linear_batch<K, MB, 4, ROT>>()));
+  HTR_CHECK_HIP(launch_kernel(k_linear_batch<K, MB, 4, ROT>, dim3(bp.S, a.m / 128), dim3(WG_THREADS), lds, st, a.qw, a.part, a.x, a.su,
+                              a.m, a.n, a.M, bp.S, a.flags, t));
   return HTR_OK;
 }
-template <int K> int launch_batch_k(const uint32_t* qw, float* part, int m, int n, int M, int flags, const LinearTail& t,
-                                    const BatchPlan& bp, hipStream_t st) {
+template <int K> int launch_batch_k(const BatchArgs& a, bool rot, const LinearTail& t, const BatchPlan& bp, hipStream_t st) {
+  if (rot) return launch_batch_v<K, 1, true>(a, t, bp, st);
   switch (bp.mb) {
-    case 1: return launch_batch_v<K, 1>(qw, part, m, n, M, flags, t, bp, st);
-    case 2: return launch_batch_v<K, 2>(qw, part, m, n, M, flags, t, bp, st);
-    case 4: return launch_batch_v<K, 4>(qw, part, m, n, M, flags, t, bp, st);
-    default: return launch_batch_v<K, 8>(qw, part, m, n, M, flags, t, bp, st);
+    case 1: return launch_batch_v<K, 1, false>(a, t, bp, st);
+    case 2: return launch_batch_v<K, 2, false>(a, t, bp, st);
+    case 4: return launch_batch_v<K, 4, false>(a, t, bp, st);
+    default: return launch_batch_v<K, 8, false>(a, t, bp, st);
   }
 }
 // nsplit bit 29: batched kernel with the split in the low bits (0 = policy); otherwise the policy decides by M
 // Tall matrices (192 row blocks and more) fill the chip without column splits, so the batched kernel needs no exchange
 // there and wins from 6 rows (65536x4096, 8 rows: 41 against 50 us; 152064x4096: 91 against 95).
-inline bool wants_batch(int M, int nsplit, int m) {
+// A matrix whose splits are four column blocks or fewer on a full grid (4096x4096: 8 splits of 4 blocks) is also ahead
+// with the batched kernel at 7 and 8 rows, when its workgroups rotate their own slices (8 rows: 9.2 against 10.4 us).
+inline bool wants_batch(int M, int nsplit, int m, int n) {
   if (nsplit > 0) return (nsplit & (1 << 29)) != 0;
-  return M >= BATCH_MIN_M || (M >= 6 && m / 128 >= 192);
+  if (M >= BATCH_MIN_M || (M >= 6 && m / 128 >= 192)) return true;
+  if (M >= 7) {
+    BatchPlan bp;
+    return make_batch_plan(m, n, M, 0, bp) && bp.rot && bp.cb <= 4 && bp.wgs >= NUM_CU;
+  }
+  return false;
 }
 
 // Rotation of all rows of x ahead of a linear launch: on the matrix unit for 16-bit rows on 16-byte boundaries, else the
@@ -2109,7 +2228,7 @@ float htr_cbscale(void) { return (float)(1.0 / __builtin_sqrt(MEAN_SQ)); }
 
 size_t htr_workspace_bytes(int m, int n, int K, int M, int nsplit) {
   if (K < 2 || K > 8 || !shape_ok(m, n) || M < 1 || M > HTR_MAX_BATCH) return 0;
-  if (wants_batch(M, nsplit, m)) {
+  if (wants_batch(M, nsplit, m, n)) {
     BatchPlan bp;
     if (!make_batch_plan(m, n, M, nsplit > 0 ? nsplit & 0xFFFFF : 0, bp)) return 0;
     return ws_need((size_t)bp.wgs * M * 128 * sizeof(float), prerot_bytes(n, M));
@@ -2125,10 +2244,10 @@ int htr_linear_plan(int m, int n, int K, int M, int nsplit, int* out6) {
   if (K < 2 || K > 8) return HTR_ERR_K;
   if (!shape_ok(m, n)) return HTR_ERR_SHAPE;
   if (M < 1 || M > HTR_MAX_BATCH) return HTR_ERR_BATCH;
-  if (wants_batch(M, nsplit, m)) {
+  if (wants_batch(M, nsplit, m, n)) {
     BatchPlan bp;
     if (!make_batch_plan(m, n, M, nsplit > 0 ? nsplit & 0xFFFFF : 0, bp)) return HTR_ERR_SPLIT;
-    out6[0] = bp.cb; out6[1] = bp.wgs; out6[2] = 1; out6[3] = 1; out6[4] = 1; out6[5] = (int)bp.lds;
+    out6[0] = bp.cb; out6[1] = bp.wgs; out6[2] = 1; out6[3] = 1; out6[4] = bp.rot ? 0 : 1; out6[5] = (int)bp.lds;
     return HTR_OK;
   }
   if (M > HTR_MAX_GROUP_ROWS) return HTR_ERR_BATCH;
@@ -2169,7 +2288,7 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
   if (((uintptr_t)qweight & 15) || ((uintptr_t)scales & 1) || ((uintptr_t)x & (x_dtype == HTR_F32 ? 3 : 1)) ||
       ((uintptr_t)y & (y_dtype == HTR_F32 ? 3 : 1)) || (bias && ((uintptr_t)bias & (y_dtype == HTR_F32 ? 3 : 1))))
     return HTR_ERR_ALIGN;
-  if (wants_batch(M, nsplit, m)) {
+  if (wants_batch(M, nsplit, m, n)) {
     BatchPlan bp;
     if (!make_batch_plan(m, n, M, nsplit > 0 ? nsplit & 0xFFFFF : 0, bp)) return HTR_ERR_SPLIT;
     const size_t need = htr_workspace_bytes(m, n, K, M, nsplit);
@@ -2186,10 +2305,14 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
     t.chunk_magic = 0;
     t.group = nullptr; t.group_prerot_stride = 0; t.group_part_stride = 0;
     hipStream_t st = (hipStream_t)stream;
-    HTR_CHECK_HIP(launch_rotation(x, (const uint8_t*)su, n, M, x_dtype, t, st));
-    float* part = (float*)((unsigned char*)workspace + WS_HEADER);
-    const int flags = x_dtype | (y_dtype << 2);
-    HTR_FOR_K(K, return launch_batch_k<KK>((const uint32_t*)qweight, part, m, n, M, flags, t, bp, st));
+    // the workgroups rotate their own activations where the plan allows it (16-bit rows on 16-byte boundaries)
+    const bool rot = bp.rot && x_dtype != HTR_F32 && ((uintptr_t)x & 15) == 0;
+    if (!rot) HTR_CHECK_HIP(launch_rotation(x, (const uint8_t*)su, n, M, x_dtype, t, st));
+    BatchArgs ba;
+    ba.qw = (const uint32_t*)qweight; ba.part = (float*)((unsigned char*)workspace + WS_HEADER); ba.x = x; ba.su = (const uint8_t*)su;
+    ba.m = m; ba.n = n; ba.M = M; ba.flags = x_dtype | (y_dtype << 2);
+    if (bp.rot && !rot) bp.lds = batch_lds_bytes(M);            // the staged kernel's layout
+    HTR_FOR_K(K, return launch_batch_k<KK>(ba, rot, t, bp, st));
     return HTR_OK;
   }
   if (M > HTR_MAX_GROUP_ROWS) return HTR_ERR_BATCH;          // an explicit chunked plan: that kernel takes up to 32 rows

@@ -102,8 +102,10 @@ unsigned long long htr_stream_capture_id(void* stream);
  * per workgroup, workgroups, row blocks that can end inside one workgroup's chunk, distinct column blocks per
  * workgroup, 1 if the activations are rotated by a launch of their own, dynamic LDS bytes}.  No reference counterpart
  * as a function; it exposes what nsplit_for / fused_nsplit decide there (htr/ops.py:31-45).
- * With 9 rows and more (6 and more for m >= 24576; library policy) the batched kernel runs instead: out6 = {column blocks per split, workgroups
- * (= row blocks x splits), 1, 1, 1, dynamic LDS bytes}.
+ * With 9 rows and more (6 and more for m >= 24576, 7 and more where a full grid has splits of at most four column blocks;
+ * library policy) the batched kernel runs instead: out6 = {column blocks per split, workgroups
+ * (= row blocks x splits), 1, 1, 1 if the activations are rotated by a launch of their own (0: up to 16 rows over at most 16 column
+ * blocks per split, where the workgroups rotate their own slices), dynamic LDS bytes}.
  * nsplit: 0 = library policy; otherwise the steps per workgroup of the chunked kernel (1 .. HTR_MAX_GROUP_ROWS rows;
  * bit 30 set: force the separate rotation launch), or, with bit 29 set, the batched kernel with that many column
  * splits in the low bits (0 = its own policy).

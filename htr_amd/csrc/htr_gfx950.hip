@@ -1346,15 +1346,16 @@ __global__ __launch_bounds__(WG_THREADS, MG <= 2 && !ROT ? 4 : 2) void k_linear_
         const int bl = 4 * q + gk;                                 // lane (p = lane / 16, j) holds elements 32 a' + 16 h + j of block 4 q + p
         const bool live_o = bl < nsteps;
         _Float16* dst = xt + (size_t)(bl * ROWS + row) * ROWH + (j >> 3) * 64 + (j & 7);
-        float lo = 0.f, hi = 0.f;
+        float lo = 0.f, hi = 0.f;                                  // sums of the rounded values: columns 0..63 | 64..127
+        const h2 ones = {(_Float16)1.f, (_Float16)1.f};
 #pragma unroll
-        for (int h = 0; h < 2; ++h)
-#pragma unroll
-          for (int a = 0; a < 4; ++a) {
-            const _Float16 hv = (_Float16)(y[h][a] * f);
-            if (live_o) dst[(2 * a + h) * 8] = hv;
-            if (a < 2) lo += (float)hv; else hi += (float)hv;       // columns 0..63 | 64..127
-          }
+        for (int h = 0; h < 2; ++h) {
+          const h2 p01 = __builtin_convertvector(f2{y[h][0] * f, y[h][1] * f}, h2);
+          const h2 p23 = __builtin_convertvector(f2{y[h][2] * f, y[h][3] * f}, h2);
+          if (live_o) { dst[(0 + h) * 8] = p01.x; dst[(2 + h) * 8] = p01.y; dst[(4 + h) * 8] = p23.x; dst[(6 + h) * 8] = p23.y; }
+          lo = __builtin_amdgcn_fdot2(p01, ones, lo, false);
+          hi = __builtin_amdgcn_fdot2(p23, ones, hi, false);
+        }
         lo += dpp_mov<0xB1>(lo); lo += dpp_mov<0x4E>(lo); lo += dpp_mov<0x141>(lo); lo += dpp_mov<0x140>(lo);
         hi += dpp_mov<0xB1>(hi); hi += dpp_mov<0x4E>(hi); hi += dpp_mov<0x141>(hi); hi += dpp_mov<0x140>(hi);
         if (live_o && j == 0) { s_xs[(bl * ROWS + row) * 2] = lo; s_xs[(bl * ROWS + row) * 2 + 1] = hi; }

@@ -1119,7 +1119,7 @@ template <int K, int MG, int P, bool ROT>
 __global__ __launch_bounds__(WG_THREADS, MG <= 2 && !ROT ? 4 : 2) void k_linear_batch(const uint32_t* __restrict__ qw, float* __restrict__ part,
                                                              const void* __restrict__ x, const uint8_t* __restrict__ su,
                                                              int m, int n, int M, int S, int flags, const LinearTail t) {
-  static_assert(!ROT || MG == 1, "the variant that rotates its own activations holds 16 rows");
+  static_assert(!ROT || MG <= 2, "the variant that rotates its own activations holds up to 32 rows");
   extern __shared__ __align__(16) unsigned char lds[];
   const int lane = threadIdx.x & 63;
   const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
@@ -1135,10 +1135,11 @@ __global__ __launch_bounds__(WG_THREADS, MG <= 2 && !ROT ? 4 : 2) void k_linear_
   // [2 column halves][M][132] partial of the workgroup.  Rows M .. 16 MG - 1 are staged like the others (they read out of
   // range: zeros), so every group of 16 rows is addressed alike.  With more than 64 rows the partial does not fit
   // behind the blocks and takes their place once the last step is done.
-  // ROT (up to 16 rows, up to 16 column blocks per split): no rotation launch; the workgroup rotates the activations
-  // of its own column blocks at the start (wave w: rows 2w and 2w + 1, four blocks per pass on the matrix unit, one
-  // power-of-two scale per row from max|x| over the split's columns) and keeps all of them in LDS, [cb blocks][16 rows]
-  // [136 halves] + [cb][16][2] sums: no staging and no barrier inside the loop.
+  // ROT (up to 16 rows over up to 16 column blocks per split, or up to 32 rows over up to 8): no rotation launch; the
+  // workgroup rotates the activations of its own column blocks at the start (wave w: rows 2 MG w .. 2 MG w + 2 MG - 1,
+  // four blocks per pass on the matrix unit, eight passes, one power-of-two scale per row from max|x| over the split's
+  // columns) and keeps all of them in LDS, [cb blocks][16 MG rows][136 halves] + [cb][16 MG][2] sums: no staging and no
+  // barrier inside the loop.
   constexpr int ROWH = BATCH_ROWH, ROWS = 16 * MG, BUFH = ROWS * ROWH;
   constexpr bool FIN_OVER_BLOCKS = MG > 4;
   _Float16* xt = (_Float16*)lds;
@@ -1185,8 +1186,9 @@ __global__ __launch_bounds__(WG_THREADS, MG <= 2 && !ROT ? 4 : 2) void k_linear_
       if (has_piece) *(u4*)(xt + q * BUFH + piece_lds[i]) = xg[set][i];
     if (has_sum) s_xs[q * 2 * ROWS + tid] = xsg[set];
   };
-  // ROT: the raw activations of this wave's two rows, eight passes of four blocks, all loads back to back
+  // ROT: the raw activations of this wave's rows, eight passes of four blocks, all loads back to back
   constexpr int RPASS = ROT ? 8 : 1;
+  constexpr int ROTR = 2 * MG, PPR = 8 / ROTR;          // rows a wave rotates, passes (of four blocks) per row
   u4 rx[RPASS];
   uint32_t rsb[RPASS];
   if constexpr (ROT) {
@@ -1195,7 +1197,7 @@ __global__ __launch_bounds__(WG_THREADS, MG <= 2 && !ROT ? 4 : 2) void k_linear_
     int xo[RPASS], so[RPASS];
 #pragma unroll
     for (int r = 0; r < RPASS; ++r) {
-      const int row = 2 * w + (r >> 2), bl = 4 * (r & 3) + ((lane & 15) >> 2);          // block within the split
+      const int row = ROTR * w + r / PPR, bl = 4 * (r % PPR) + ((lane & 15) >> 2);      // block within the split
       const int col = (c_begin + bl) * 128 + 32 * (lane & 3) + 8 * (lane >> 4);
       const bool live = row < M && bl < nsteps;
       xo[r] = live ? (row * n + col) * 2 : OUT_OF_RANGE;
@@ -1319,15 +1321,15 @@ __global__ __launch_bounds__(WG_THREADS, MG <= 2 && !ROT ? 4 : 2) void k_linear_
   const int hist = history_lane_byteaddr(lane);
   DecodedStep<K> cur;
   if constexpr (ROT) {
-    // ---- rotation of this wave's two rows.  Row scale from the raw values: |H128 x| / sqrt(128) <= sqrt(128) max|x|.
+    // ---- rotation of this wave's rows.  Row scale from the raw values: |H128 x| / sqrt(128) <= sqrt(128) max|x|.
     const bool is_bf16 = (flags & 3) == HTR_BF16;
     const int j = lane & 15, gk = lane >> 4;
 #pragma unroll
-    for (int rr = 0; rr < 2; ++rr) {
+    for (int rr = 0; rr < ROTR; ++rr) {
       uint32_t m16 = 0u;
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const uint32_t d[4] = {rx[4 * rr + q].x, rx[4 * rr + q].y, rx[4 * rr + q].z, rx[4 * rr + q].w};
+      for (int q = 0; q < PPR; ++q) {
+        const uint32_t d[4] = {rx[PPR * rr + q].x, rx[PPR * rr + q].y, rx[PPR * rr + q].z, rx[PPR * rr + q].w};
 #pragma unroll
         for (int k = 0; k < 4; ++k) m16 = max(m16, max(d[k] & 0x7FFFu, (d[k] >> 16) & 0x7FFFu));
       }
@@ -1336,13 +1338,13 @@ __global__ __launch_bounds__(WG_THREADS, MG <= 2 && !ROT ? 4 : 2) void k_linear_
       if (amax != amax) amax = __uint_as_float(0x7F800000u);      // a NaN anywhere: treat the row as unbounded (scale 1)
       const int e = scale_exponent(amax);
       const float f = pow2f(-e) * INV_SQRT128;
-      const int row = 2 * w + rr;
+      const int row = ROTR * w + rr;
       if (lane == 0) s_sc[row] = row < M ? pow2f(e) : 0.f;
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
+      for (int q = 0; q < PPR; ++q) {
         if (4 * q >= nsteps) continue;                             // uniform: none of the pass's blocks exists
         float y[2][4];
-        rotate4_mfma(rx[4 * rr + q], rsb[4 * rr + q], is_bf16, lane, y);
+        rotate4_mfma(rx[PPR * rr + q], rsb[PPR * rr + q], is_bf16, lane, y);
         const int bl = 4 * q + gk;                                 // lane (p = lane / 16, j) holds elements 32 a' + 16 h + j of block 4 q + p
         const bool live_o = bl < nsteps;
         _Float16* dst = xt + (size_t)(bl * ROWS + row) * ROWH + (j >> 3) * 64 + (j & 7);
@@ -2105,8 +2107,9 @@ template <int K> int launch_linear_k(const LinearLaunch& a, bool prerot, int mb,
 
 // ---- batched kernel: split S of the column blocks per row block
 struct BatchPlan { int S, cb, wgs, mb, rot; size_t lds; };
-constexpr int BATCH_ROT_MAX_M = 16;      // rows and column blocks per split up to which a workgroup of the batched kernel
-constexpr int BATCH_ROT_MAX_CB = 16;     // rotates its own activations (256 pairs, eight passes per wave) instead of a rotation launch
+// rows x column blocks per split up to which a workgroup of the batched kernel rotates its own activations (256 pairs,
+// eight passes per wave) instead of a rotation launch: 16 x 16 or 32 x 8
+inline bool batch_rot_fits(int M, int cb) { return (M <= 16 && cb <= 16) || (M <= 32 && cb <= 8); }
 constexpr int BATCH_MIN_M = 9;      // rows from which the library policy takes the batched kernel on every shape
 inline int batch_groups(int M) { return M <= 16 ? 1 : (M <= 32 ? 2 : (M <= 64 ? 4 : 8)); }   // groups of 16 activation rows
 inline size_t batch_lds_bytes(int M) {
@@ -2134,12 +2137,13 @@ inline bool make_batch_plan(int m, int n, int M, int want_S, BatchPlan& bp) {
     if (want_S > 0 && S != want_S) continue;
     bp.S = S; bp.cb = cb; bp.wgs = rbs * S; found = true;
   }
-  // Up to 16 rows over at most 16 column blocks per split, one workgroup per CU: every workgroup rotates its own slice
-  // (measured on MI355X, K4, 16 rows: see the launch comment in htr_linear).  HTR_BATCH_ROT=0 switches it off.
+  // Few rows over few column blocks per split, one workgroup per CU: every workgroup rotates its own slice.
+  // HTR_BATCH_ROT=0 switches it off.
   static const bool rot_on = getenv("HTR_BATCH_ROT") == nullptr || atoi(getenv("HTR_BATCH_ROT")) != 0;
-  if (found && rot_on && M <= BATCH_ROT_MAX_M && bp.cb <= BATCH_ROT_MAX_CB && bp.wgs <= NUM_CU) {
+  if (found && rot_on && batch_rot_fits(M, bp.cb) && bp.wgs <= NUM_CU) {
+    const int rows = 16 * bp.mb;
     bp.rot = 1;
-    bp.lds = (size_t)bp.cb * 16 * BATCH_ROWH * 2 + (size_t)bp.cb * 32 * 4 + 16 * 4 + (size_t)2 * M * BATCH_FIN_STRIDE * 4;
+    bp.lds = (size_t)bp.cb * rows * BATCH_ROWH * 2 + (size_t)bp.cb * 2 * rows * 4 + rows * 4 + (size_t)2 * M * BATCH_FIN_STRIDE * 4;
   }
   return found;
 }
@@ -2153,7 +2157,7 @@ template <int K, int MB, bool ROT> int launch_batch_v(const BatchArgs& a, const 
   return HTR_OK;
 }
 template <int K> int launch_batch_k(const BatchArgs& a, bool rot, const LinearTail& t, const BatchPlan& bp, hipStream_t st) {
-  if (rot) return launch_batch_v<K, 1, true>(a, t, bp, st);
+  if (rot) return bp.mb == 1 ? launch_batch_v<K, 1, true>(a, t, bp, st) : launch_batch_v<K, 2, true>(a, t, bp, st);
   switch (bp.mb) {
     case 1: return launch_batch_v<K, 1, false>(a, t, bp, st);
     case 2: return launch_batch_v<K, 2, false>(a, t, bp, st);

@@ -88,12 +88,12 @@ def test_launch_plan_is_consistent(L, m, n, M):
         batched = forced[4] == 0 and forced[0] <= 4 and forced[1] >= 256
     if batched:
         # batched kernel: `chunk` column blocks per split, S = ceil(nblk / chunk) splits per row block, no empty split;
-        # activations rotated ahead, except up to 16 rows over at most 16 column blocks per split on a grid of one
-        # workgroup per CU, where every workgroup rotates and keeps its own slice (more LDS)
+        # activations rotated ahead, except up to 16 rows over at most 16 column blocks per split (32 rows over 8) on a
+        # grid of one workgroup per CU, where every workgroup rotates and keeps its own slice (more LDS)
         S = -(-nblk // chunk)
-        in_kernel = M <= 16 and chunk <= 16 and wgs <= 256
+        in_kernel = ((M <= 16 and chunk <= 16) or (M <= 32 and chunk <= 8)) and wgs <= 256
         assert wgs == rbs * S and (S - 1) * chunk < nblk and prerot == (0 if in_kernel else 1)
-        assert lds <= (96 if in_kernel else 64 if M <= 32 else 140) * 1024
+        assert lds <= (112 if in_kernel else 64 if M <= 32 else 140) * 1024
         assert S <= 8 and (wgs <= 256 or S == 1)                                 # the grid fits the chip, at most 8 splits
         # an explicit split is honoured (bit 29 selects the batched kernel)
         assert L.htr_linear_plan(m, n, 4, M, (1 << 29) | 1, out) == 0 and out[0] == nblk and out[1] == rbs

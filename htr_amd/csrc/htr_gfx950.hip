@@ -1092,11 +1092,12 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
 }
 
 // ------------------------------------------------------------------------------------------------ batched linear
-// Variant for 8 .. 32 activation rows.  With that many rows the rotated activations of a whole chunk no longer fit in
+// Variant for 9 .. 128 activation rows.  With that many rows the rotated activations of a whole chunk no longer fit in
 // LDS next to useful chunk lengths, and short chunks mean that every workgroup copies a large activation slice and
 // hands over a large partial for little weight traffic.  Here a workgroup owns one 128-row block and 1/S of its
-// column blocks (grid = S x row blocks), and the activations (rotated ahead by k_rotate) are staged through LDS one
-// 128-column block at a time, double-buffered, one barrier per step.  The split S along the columns is only as large
+// column blocks (grid = S x row blocks), and the activations (rotated ahead by a launch of their own) are staged through
+// LDS one 128-column block at a time, double-buffered, one barrier per step; with few rows over few column blocks the
+// workgroup rotates its own slice instead and keeps it in LDS (ROT, below).  The split S along the columns is only as large
 // as filling the chip needs; S = 1 needs no exchange.
 //   wave    = two adjacent 16-row strips (pair sp = w / 2) x one half (ch = w % 2) of the block's columns: 2 x 4 tiles
 //             per step, two runs of 128 K contiguous bytes

@@ -543,3 +543,22 @@ def test_seeded_random_cases_through_the_c_abi(dev, oracle):
                 assert not np.any(got[r]), (it, r)
             else:
                 assert np.abs(got[r] - ref[r]).max() <= tols[ydt] * den, (it, r, float(np.abs(got[r] - ref[r]).max() / den))
+
+
+@pytest.mark.parametrize("M,S", [(12, 1), (16, 1), (16, 2), (32, 1), (32, 4), (10, 8)])
+def test_batched_kernel_with_explicit_splits(dev, oracle, M, S, monkeypatch):
+    """The batched kernel with an explicit number of column splits (nsplit bit 29): one split of 32 column blocks is more
+    than a workgroup rotates and keeps by itself, so those cases take the rotation launch and the staged blocks also at
+    few rows; the short splits take the in-kernel rotation.  Same result either way."""
+    import ctypes
+    from htr_amd import _native, ops
+    print(f"batched kernel, explicit splits M={M} S={S}", flush=True)
+    m, n = 512, 4096
+    out = (ctypes.c_int * 6)()
+    assert _native.lib().htr_linear_plan(m, n, 4, M, (1 << 29) | S, out) == 0
+    cb = out[0]
+    assert cb == 32 // S and out[4] == (0 if (M <= 16 and cb <= 16) or cb <= 8 else 1)
+    qw, sc, su, sv, x = _case(m, n, 4, M, 5200 + 10 * M + S)
+    monkeypatch.setattr(ops, "NSPLIT", (1 << 29) | S)
+    y = ops.linear_f32out(x.to(dev), *[t.to(dev) for t in (qw, sc, su, sv)]).cpu().numpy()
+    assert _rel(y, _ref(oracle, qw, sc, su, sv, x)) <= REL_TOL

@@ -136,7 +136,9 @@ def make_signs(n, m, seed, index, shared_su):
 
 def prep_H(H, W, damp=0.01):
     """Dead input columns get a unit diagonal and zero weights; the diagonal is damped by damp * mean(diag)
-    (htr/encode.py:35-42).  float64."""
+    (htr/encode.py:35-42).  float64.  The order of these float64 operations (dead columns first, then the damping added
+    to the whole matrix as damp * mean * I) is kept as the reference has it: the encoder's fixture is matched bit for
+    bit, and damping the diagonal in place, or before the dead columns are fixed, rounds differently."""
     H = H.clone().double()
     dead = torch.diag(H) == 0
     H[dead, dead] = 1.0

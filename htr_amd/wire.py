@@ -25,9 +25,14 @@ def cbscale():
 
 
 def gen_values(states):
-    """Integer codebook value v(s) for int64 states of any shape (htr/wire.py:10-13)."""
-    x = (states.long() * GEN_A + GEN_B) & 0xFFFFFFFF
-    return ((x & 0xFF) + ((x >> 8) & 0xFF) + ((x >> 16) & 0xFF) + ((x >> 24) & 0xFF)) - 510
+    """Integer codebook value v(s) for integer states of any shape (htr/wire.py:10-13): the generator word
+    s * A + B is reduced mod 2^32 and its four bytes are summed; the sum of four uniform bytes has mean 510."""
+    word = torch.remainder(states.to(torch.int64) * GEN_A + GEN_B, 1 << 32)
+    total = torch.zeros_like(word)
+    for _ in range(4):
+        total += torch.remainder(word, 256)
+        word = word // 256
+    return total - 510
 
 
 _CACHE = {}
@@ -43,18 +48,24 @@ def codebook_f32(device="cpu"):
 
 
 def hadamard(n, device="cpu"):
-    """Sylvester Hadamard matrix / sqrt(n), built in float64 and rounded once to float32 (htr/wire.py:80-87)."""
+    """Sylvester Hadamard matrix / sqrt(n) (htr/wire.py:80-87): entry (i, j) is (-1)^popcount(i & j); the division is
+    done in float64 and rounded once to float32, which is what the reference's recursion yields as well."""
     key = ("had", n, str(device))
     if key not in _CACHE:
-        h = torch.ones(1, 1, dtype=torch.float64)
-        while h.shape[0] < n:
-            h = torch.cat([torch.cat([h, h], 1), torch.cat([h, -h], 1)], 0)
-        _CACHE[key] = (h / math.sqrt(n)).float().to(device)
+        i = torch.arange(n, dtype=torch.int64)
+        both = i[:, None] & i[None, :]
+        parity = torch.zeros_like(both)
+        while bool(both.any()):
+            parity ^= both & 1
+            both = both >> 1
+        _CACHE[key] = ((1.0 - 2.0 * parity.double()) / math.sqrt(n)).float().to(device)
     return _CACHE[key]
 
 
 def blk_had_cols_T(W, bs=RHT_BLOCK):
-    """Every block of bs consecutive columns of W times H (htr/wire.py:90-92)."""
+    """Every block of bs consecutive columns of W times H (htr/wire.py:90-92).  The batched float32 matmul, in this
+    form, is the contract: the reference's encoder fixture (What) is reproduced bit for bit only with torch's own
+    summation order."""
     m, n = W.shape
     return (W.reshape(m, n // bs, bs) @ hadamard(bs, W.device)).reshape(m, n)
 
@@ -83,7 +94,8 @@ def dequant_Q(qweight, scales):
 
 def dequant(qweight, scales, su8, sv8):
     """Original-basis W [m, n] float32 = Sv . Ho . Q . Hi . Su with torch, in the reference's order of operations
-    (htr/wire.py:105-113)."""
+    (htr/wire.py:105-113): rows first, then columns, then both signs.  The order is kept on purpose; any other one
+    rounds differently and no longer matches the reference's What fixture bit for bit."""
     Q = dequant_Q(qweight, scales)
     m, n = Q.shape
     su = unpack_signs(su8, n).to(Q.device)
@@ -101,9 +113,11 @@ def pack_signs(s):
 
 
 def unpack_signs(u8, N):
-    """uint8 [N/8] -> float32 +-1 [N] (htr/wire.py:72-74)."""
-    bits = (u8.view(-1, 1).to(torch.int32) >> torch.arange(8, dtype=torch.int32, device=u8.device)) & 1
-    return 1.0 - 2.0 * bits.reshape(-1)[:N].float()
+    """uint8 [N/8] -> float32 +-1 [N]: element j is -1 where bit j % 8 of byte j / 8 is set (htr/wire.py:72-74)."""
+    j = torch.arange(N, device=u8.device)
+    byte = u8.reshape(-1).to(torch.int64)[j // 8]
+    minus = torch.remainder(byte // (1 << (j % 8)), 2) == 1
+    return torch.where(minus, -1.0, 1.0).to(torch.float32)
 
 
 def pack_states(states, K):
@@ -111,12 +125,15 @@ def pack_states(states, K):
     B, T = states.shape
     if T != 256 or not 2 <= K <= 8:
         raise ValueError("pack_states wants [B, 256] states and 2 <= K <= 8")
-    b = states.long() & ((1 << K) - 1)
-    sh = torch.arange(K - 1, -1, -1, device=states.device)
-    bits = ((b[:, :, None] >> sh) & 1).reshape(B, 8 * K, 32)
-    wsh = torch.arange(31, -1, -1, device=states.device)
-    words = (bits << wsh).sum(-1)
-    return torch.where(words >= 2 ** 31, words - 2 ** 32, words).to(torch.int32)
+    # the stream is the states' low K bits one after the other; bit p of it (MSB first) belongs to state p / K and is
+    # that state's bit K - 1 - p % K; 32 consecutive stream bits make one big-endian word
+    p = torch.arange(256 * K, device=states.device)
+    fresh = torch.remainder(states.to(torch.int64), 1 << K)
+    stream = torch.remainder(fresh[:, p // K] // (1 << (K - 1 - p % K)), 2)
+    place = 1 << (31 - p % 32)
+    words = torch.zeros(B, 8 * K, dtype=torch.int64, device=states.device)
+    words.index_add_(1, p // 32, stream * place)
+    return (words - (words >> 31) * (1 << 32)).to(torch.int32)          # two's complement view of the uint32 value
 
 
 def bits_of(qweight):

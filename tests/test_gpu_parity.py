@@ -456,6 +456,58 @@ def test_moe_64_experts_grouped(dev, oracle):
     assert _rel(y, y_ref) <= 4e-3, _rel(y, y_ref)
 
 
+def test_moe_expert_shapes_grouped_per_stage(dev, oracle):
+    """The grouped launch at the real expert shapes, each stage on its own at the single-linear bar: gate_up 2816x2048 and
+    down 2048x1408 (K4) of three experts with ragged token counts, against the float64 oracle, 1e-3 per linear."""
+    from htr_amd import ops, wire
+    print("moe expert shapes, per stage", flush=True)
+    H, F = 2048, 1408
+    rows = [1, 6, 3]
+    gate_up = [wire.synth_linear(2 * F, H, 4, 7000 + e) for e in range(3)]
+    down = [wire.synth_linear(H, F, 4, 7100 + e) for e in range(3)]
+    xs = [wire.synth_activation(r, H, 7200 + e) for e, r in enumerate(rows)]
+    hs = [wire.synth_activation(r, F, 7300 + e) for e, r in enumerate(rows)]
+    for name, ws, ins in (("gate_up", gate_up, xs), ("down", down, hs)):
+        got = ops.linear_grouped([t.to(dev) for t in ins], [tuple(t.to(dev) for t in w) for w in ws], out_dtype=torch.float32)
+        for e, r in enumerate(rows):
+            ref = _ref(oracle, *ws[e], ins[e])
+            assert tuple(got[e].shape) == ref.shape
+            assert _rel(got[e].cpu().numpy(), ref) <= REL_TOL, (name, e, _rel(got[e].cpu().numpy(), ref))
+
+
+def test_reference_encoded_streams_decode_on_the_gpu(dev, oracle):
+    """The tensors the reference's own encoder wrote (tests/golden/encode_small.npz: qweight, scales, su, sv and its
+    reconstruction What, the objects of tests/test_release.py:53-73 of the reference) through every decode entry point:
+    integer decode and float32 Q bit-exact against the oracle; Q rotated back with torch's block-Hadamard products equals
+    What bit for bit (as wire.dequant does on the CPU); bf16 W within bf16 rounding of What; x @ What^T within 1e-3."""
+    import os
+    from htr_amd import ops, wire
+    print("reference-encoded streams", flush=True)
+    gold = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "encode_small.npz"))
+    for tag in ("a", "b0", "b1"):
+        qw = torch.from_numpy(gold[f"{tag}_qweight"])
+        sc = torch.from_numpy(gold[f"{tag}_scales_f16bits"].view(np.float16))
+        su, sv = torch.from_numpy(gold[f"{tag}_su"]), torch.from_numpy(gold[f"{tag}_sv"])
+        what = gold[f"{tag}_What"]
+        m, n = what.shape
+        d = [t.to(dev) for t in (qw, sc, su, sv)]
+        assert np.array_equal(ops.decode_raw(d[0]).cpu().numpy(), oracle.c_decode_raw(qw.numpy())), tag
+        q = ops.dequant_q(d[0], d[1])
+        assert np.array_equal(q.cpu().numpy().view(np.uint32), oracle.c_dequant_q(qw.numpy(), sc.numpy()).view(np.uint32)), tag
+        # the reference's own order of operations on the device's Q, on the CPU (its matmul is the fixture's)
+        qc = q.cpu()
+        w = wire.blk_had_cols_T(wire.blk_had_cols_T(qc.T.contiguous()).T.contiguous())
+        w = (w * wire.unpack_signs(sv, m)[:, None] * wire.unpack_signs(su, n)[None, :]).contiguous()
+        assert np.array_equal(w.numpy(), what), tag
+        wb = ops.dequant_w(*d).float().cpu().numpy()
+        assert np.all(np.abs(wb - what) <= 2.0 ** -8 * np.abs(what) + 4e-6 * np.abs(what).max()), tag
+        for M in (1, 5):
+            x = wire.synth_activation(M, n, 4242 + M)
+            y = ops.linear_f32out(x.to(dev), *d).cpu().numpy()
+            ref = x.float().numpy().astype(np.float64) @ what.astype(np.float64).T
+            assert _rel(y, ref) <= REL_TOL, (tag, M, _rel(y, ref))
+
+
 def test_lm_head_shape(dev, oracle):
     from htr_amd import ops
     print("lm_head 152064x4096", flush=True)

@@ -28,6 +28,7 @@ SIGNATURES = {
     "htr_cbscale": (ctypes.c_float, []),
     "htr_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "htr_linear_plan": (_i, [_i, _i, _i, _i, _i, ctypes.POINTER(ctypes.c_int)]),
+    "htr_plan_device_override": (_i, [_i, ctypes.c_long]),
     "htr_linear": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
     "htr_linear_static": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
     "htr_grouped_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),

@@ -592,6 +592,7 @@ __device__ __forceinline__ uint32_t load_status(const uint32_t* status) {
   return __hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 constexpr int FLAG_LANES = 1 << 4;     // kernel flag: chunk ids are dealt to the XCDs in eight lanes (see k_linear)
+constexpr int FLAG_LAST_FINISHES = 1 << 5;   // batched kernel: the last split of a row block finishes all of its rows (see there)
 constexpr int FLAG_LANE_LEN_SHIFT = 8; // with FLAG_LANES: grid / 8 in the bits from here up (no read of the hidden grid-size argument)
 
 template <int K, int MB, int P, int D, bool PREROT, int RP>
@@ -1220,7 +1221,9 @@ __global__ __launch_bounds__(WG_THREADS, MG <= 2 && !ROT ? 4 : 2) void k_linear_
   // row constants of the output side (scale, sign, bias of rows lane and lane + 64), requested ahead of the weight stream by
   // the workgroups that finish rows of the row block, so that they have long arrived when they are needed
   const int RG = (M + 7) >> 3;               // groups of eight activation rows
-  const bool spread = M > 16 || (M > 8 && S > 2);   // the splits share the output side (below)
+  // the splits share the output side (below), unless the host found that the grid does not fit the chip at once: splits
+  // that wait for each other must all be resident, a last split that waits for the earlier ones need not be
+  const bool spread = (M > 16 || (M > 8 && S > 2)) && !(flags & FLAG_LAST_FINISHES);
   const bool finisher = spread ? s_idx < RG : s_idx == S - 1;
   const int r0 = rb * 128 + lane, r1 = r0 + 64;
   uint32_t raw_sc0 = 0u, raw_sc1 = 0u, raw_sv0 = 0u, raw_sv1 = 0u, raw_b0 = 0u, raw_b1 = 0u;   // bits only: converted at the end
@@ -1444,8 +1447,8 @@ __global__ __launch_bounds__(WG_THREADS, MG <= 2 && !ROT ? 4 : 2) void k_linear_
   // (group rg = rows 8 rg .. 8 rg + 7, one row per wave): split rg mod S finishes group rg, every other split leaves
   // its partial of those rows in its slot.  So the output side of many rows is spread over the splits instead of
   // falling to one workgroup (32 rows on 4096x14336, 8 splits: 23.0 -> 19.7 us; 128 rows: 56.6 -> 38.5).  The
-  // workgroups of one row block are neighbours in dispatch order and the grid fits the chip, so they run together; the
-  // wait is bounded all the same.  Up to 8 rows (one group), and up to 16 rows with two splits, the last split
+  // workgroups of one row block are neighbours in dispatch order and the grid fits the chip (the host checks it against
+  // the device's CU count and otherwise sets FLAG_LAST_FINISHES), so they run together; the wait is bounded all the same.  Up to 8 rows (one group), and up to 16 rows with two splits, the last split
   // finishes everything, as in k_linear: two workgroups that wait for each other cost 0.3 us more than one that waits.
   for (int rg = 0, owner = spread ? 0 : S - 1; rg < RG; ++rg, owner = !spread ? owner : (owner + 1 == S ? 0 : owner + 1)) {
     const int mrow = 8 * rg + w;
@@ -1915,7 +1918,7 @@ __global__ __launch_bounds__(256) void k_workspace_init(u4* __restrict__ ws, siz
 
 // ------------------------------------------------------------------------------------------------ host side
 thread_local int g_last_hip_error = 0;
-int g_spin_limit = 1 << 20;     // polls (about a microsecond each) before a finishing workgroup gives up
+std::atomic<int> g_spin_limit{1 << 20};     // polls (about a microsecond each) before a finishing workgroup gives up
 
 struct Plan { int chunk, wgs, segfin, nbl, mb, prerot; size_t lds; };
 
@@ -1934,7 +1937,35 @@ inline size_t ws_half(size_t workspace_bytes) { return workspace_bytes / 2 / 256
 // bytes of the pre-rotated activations, their block sums and the row scales
 inline size_t prerot_bytes(int n, int M) { return align256((size_t)M * n * 2) + align256((size_t)M * (n / 128) * 16) + align256((size_t)M * 4); }
 
-constexpr int NUM_CU = 256;
+// ---- facts of the device the plans are made for: compute units and LDS bytes per compute unit, read once per device
+// (the current one) from the runtime; an unpartitioned MI355X (256 CUs, 160 KB) where no device can be asked (plans
+// computed on a machine without a GPU).  htr_plan_device_override replaces them for every device (tests, tuning).
+struct DeviceFacts { int cus; size_t lds; };
+constexpr int MAX_DEVICES = 64;
+constexpr DeviceFacts MI355X_FACTS = {256, 160 * 1024};
+std::atomic<int> g_override_cus{0};
+std::atomic<long> g_override_lds{0};
+inline DeviceFacts device_facts() {
+  static DeviceFacts table[MAX_DEVICES];
+  static std::atomic<uint64_t> known{0};
+  const int ov = g_override_cus.load(std::memory_order_acquire);
+  if (ov > 0) return DeviceFacts{ov, (size_t)g_override_lds.load(std::memory_order_acquire)};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) { (void)hipGetLastError(); return MI355X_FACTS; }
+  if (dev < 0 || dev >= MAX_DEVICES) return MI355X_FACTS;
+  const uint64_t bit = (uint64_t)1 << dev;
+  if (known.load(std::memory_order_acquire) & bit) return table[dev];
+  int cus = 0, lds = 0;
+  if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1 ||
+      hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerMultiprocessor, dev) != hipSuccess || lds < 64 * 1024) {
+    (void)hipGetLastError();
+    return MI355X_FACTS;
+  }
+  table[dev] = DeviceFacts{cus, (size_t)lds};        // two threads racing here store the same values
+  known.fetch_or(bit, std::memory_order_release);
+  return table[dev];
+}
+inline int num_cu() { return device_facts().cus; }
 constexpr int MAX_ROW_BLOCKS = 16384;
 constexpr int MAX_CHUNK = 4096;
 // the kernel divides step indices by n / 128 with a 40-bit reciprocal: exact while indices stay below 2^24
@@ -1968,7 +1999,7 @@ inline bool plan_for_chunk(int m, int n, int M, int chunk, Plan& pl) {
 // throughput bound, proportional to the load of the fullest CU, plus a set-up per workgroup); a penalty for chunks
 // that do not tile the rows of column blocks; the extra launch of a pre-rotation; and the growth of all per-step work
 // with the number of activation rows.
-inline bool search_plan(int m, int n, int M, int nsplit, Plan& pl) {
+inline bool search_plan(int m, int n, int M, int nsplit, int cus, Plan& pl) {
   const int nblk = n / 128, rbs = m / 128;
   const long vtotal = (long)rbs * nblk;
   pl.mb = M <= 8 ? 1 : (M <= 16 ? 2 : 4);
@@ -1978,7 +2009,7 @@ inline bool search_plan(int m, int n, int M, int nsplit, Plan& pl) {
     if (ok && (nsplit & (1 << 30))) pl.prerot = 1;
     return ok;
   }
-  if (vtotal >= (long)64 * NUM_CU && nblk <= 64 && plan_for_chunk(m, n, M, nblk, pl)) return true;
+  if (vtotal >= (long)64 * cus && nblk <= 64 && plan_for_chunk(m, n, M, nblk, pl)) return true;
   const double rows = M <= 8 ? 1.0 + 0.06 * (M - 1) : (M <= 16 ? 2.2 : 6.5);
   double best = 1e30;
   bool found = false;
@@ -1987,7 +2018,7 @@ inline bool search_plan(int m, int n, int M, int nsplit, Plan& pl) {
     Plan c;
     c.mb = pl.mb;
     if (!plan_for_chunk(m, n, M, chunk, c)) continue;
-    const double fill = (double)c.wgs / NUM_CU;
+    const double fill = (double)c.wgs / cus;
     const bool aligned = (nblk % chunk == 0) || (chunk % nblk == 0);
     const int contributors = chunk >= nblk ? 1 : (nblk + chunk - 1) / chunk;
     const double steps = chunk * (aligned ? 1.0 : 1.06 + 0.04 * (M - 1));
@@ -2007,16 +2038,17 @@ inline bool search_plan(int m, int n, int M, int nsplit, Plan& pl) {
 }
 
 // The search above walks every chunk length (up to 4096 of them): tens of microseconds on the host, more than the launch
-// it plans.  Plans depend only on (m, n, M, nsplit), so the last 64 distinct ones are kept.
+// it plans.  Plans depend only on (m, n, M, nsplit) and the device's CU count, so the last 64 distinct ones are kept.
 inline bool make_plan(int m, int n, int M, int nsplit, Plan& pl) {
-  struct Entry { int m, n, M, nsplit; bool ok; Plan pl; };
+  const int cus = num_cu();
+  struct Entry { int m, n, M, nsplit, cus; bool ok; Plan pl; };
   static Entry cache[64];
   static int filled = 0, next = 0;
   static std::atomic_flag busy = ATOMIC_FLAG_INIT;
   while (busy.test_and_set(std::memory_order_acquire)) {}
   for (int i = 0; i < filled; ++i) {
     const Entry& e = cache[i];
-    if (e.m == m && e.n == n && e.M == M && e.nsplit == nsplit) {
+    if (e.m == m && e.n == n && e.M == M && e.nsplit == nsplit && e.cus == cus) {
       const bool ok = e.ok;
       pl = e.pl;
       busy.clear(std::memory_order_release);
@@ -2025,10 +2057,10 @@ inline bool make_plan(int m, int n, int M, int nsplit, Plan& pl) {
   }
   busy.clear(std::memory_order_release);
   Plan found = {};
-  const bool ok = search_plan(m, n, M, nsplit, found);
+  const bool ok = search_plan(m, n, M, nsplit, cus, found);
   while (busy.test_and_set(std::memory_order_acquire)) {}
   Entry& e = cache[next];
-  e.m = m; e.n = n; e.M = M; e.nsplit = nsplit; e.ok = ok; e.pl = found;
+  e.m = m; e.n = n; e.M = M; e.nsplit = nsplit; e.cus = cus; e.ok = ok; e.pl = found;
   next = (next + 1) % 64;
   if (filled < 64) ++filled;
   busy.clear(std::memory_order_release);
@@ -2037,13 +2069,13 @@ inline bool make_plan(int m, int n, int M, int nsplit, Plan& pl) {
 }
 
 // The dispatcher places workgroups wherever resources allow, not evenly: with 512 equal workgroups some CUs receive
-// three and others one, and the kernel ends with the most loaded CU.  Requesting 1/k of a CU's 160 KB of LDS per
+// three and others one, and the kernel ends with the most loaded CU.  Requesting 1/k of a CU's LDS (160 KB on MI355X) per
 // workgroup (k = workgroups per CU when spread evenly) makes exactly k fit, so the spread is even.
-constexpr size_t CU_LDS_BYTES = 160 * 1024;
 inline size_t balanced_lds_request(size_t needed, int grid) {
-  const int k = (grid + NUM_CU - 1) / NUM_CU;
+  const DeviceFacts df = device_facts();
+  const int k = (grid + df.cus - 1) / df.cus;
   if (k > 4) return needed;
-  const size_t share = (CU_LDS_BYTES / k) / 1024 * 1024 - 1024;
+  const size_t share = (df.lds / k) / 1024 * 1024 - 1024;
   return share > needed ? share : needed;
 }
 
@@ -2107,7 +2139,7 @@ template <int K> int launch_linear_k(const LinearLaunch& a, bool prerot, int mb,
 }
 
 // ---- batched kernel: split S of the column blocks per row block
-struct BatchPlan { int S, cb, wgs, mb, rot; size_t lds; };
+struct BatchPlan { int S, cb, wgs, mb, rot, last_finishes; size_t lds; };
 // rows x column blocks per split up to which a workgroup of the batched kernel rotates its own activations (256 pairs,
 // eight passes per wave) instead of a rotation launch: 16 x 16 or 32 x 8
 inline bool batch_rot_fits(int M, int cb) { return (M <= 16 && cb <= 16) || (M <= 32 && cb <= 8); }
@@ -2129,7 +2161,8 @@ inline bool make_batch_plan(int m, int n, int M, int want_S, BatchPlan& bp) {
   // rows: 39 against 48).  So: the largest split that keeps the grid within the CU count, among the splits that leave
   // no column range empty, and at most 8 of them (the output side requests the slots of up to eight other splits in
   // one go; 1024x4096 and 2048x4096 at 8..32 rows: 8 splits 11..12 us, 16 splits 11..16, 32 splits 14..22).
-  const int by_cus = NUM_CU / rbs > 1 ? NUM_CU / rbs : 1;
+  const int cus = num_cu();
+  const int by_cus = cus / rbs > 1 ? cus / rbs : 1;
   const int limit = want_S > 0 ? want_S : (by_cus < 8 ? by_cus : 8);
   bool found = false;
   for (int S = 1; S <= nblk && S <= limit; ++S) {
@@ -2138,10 +2171,14 @@ inline bool make_batch_plan(int m, int n, int M, int want_S, BatchPlan& bp) {
     if (want_S > 0 && S != want_S) continue;
     bp.S = S; bp.cb = cb; bp.wgs = rbs * S; found = true;
   }
+  // Splits that finish rows for each other wait for each other, which is only safe while every workgroup of the grid is
+  // resident at once: one workgroup per CU at most.  A larger grid (an explicit split, a device with fewer CUs than the
+  // policy assumed) falls back to the last split finishing everything: it waits only for workgroups dispatched before it.
+  bp.last_finishes = found && bp.wgs > cus ? 1 : 0;
   // Few rows over few column blocks per split, one workgroup per CU: every workgroup rotates its own slice.
   // HTR_BATCH_ROT=0 switches it off.
   static const bool rot_on = getenv("HTR_BATCH_ROT") == nullptr || atoi(getenv("HTR_BATCH_ROT")) != 0;
-  if (found && rot_on && batch_rot_fits(M, bp.cb) && bp.wgs <= NUM_CU) {
+  if (found && rot_on && batch_rot_fits(M, bp.cb) && bp.wgs <= cus) {
     const int rows = 16 * bp.mb;
     bp.rot = 1;
     bp.lds = (size_t)bp.cb * rows * BATCH_ROWH * 2 + (size_t)bp.cb * 2 * rows * 4 + rows * 4 + (size_t)2 * M * BATCH_FIN_STRIDE * 4;
@@ -2176,7 +2213,7 @@ inline bool wants_batch(int M, int nsplit, int m, int n) {
   if (M >= BATCH_MIN_M || (M >= 6 && m / 128 >= 192)) return true;
   if (M >= 7) {
     BatchPlan bp;
-    return make_batch_plan(m, n, M, 0, bp) && bp.rot && bp.cb <= 4 && bp.wgs >= NUM_CU;
+    return make_batch_plan(m, n, M, 0, bp) && bp.rot && bp.cb <= 4 && bp.wgs >= num_cu();
   }
   return false;
 }
@@ -2253,7 +2290,7 @@ int htr_linear_plan(int m, int n, int K, int M, int nsplit, int* out6) {
   if (wants_batch(M, nsplit, m, n)) {
     BatchPlan bp;
     if (!make_batch_plan(m, n, M, nsplit > 0 ? nsplit & 0xFFFFF : 0, bp)) return HTR_ERR_SPLIT;
-    out6[0] = bp.cb; out6[1] = bp.wgs; out6[2] = 1; out6[3] = 1; out6[4] = bp.rot ? 0 : 1; out6[5] = (int)bp.lds;
+    out6[0] = bp.cb; out6[1] = bp.wgs; out6[2] = bp.last_finishes ? 0 : 1; out6[3] = bp.S; out6[4] = bp.rot ? 0 : 1; out6[5] = (int)bp.lds;
     return HTR_OK;
   }
   if (M > HTR_MAX_GROUP_ROWS) return HTR_ERR_BATCH;
@@ -2263,7 +2300,15 @@ int htr_linear_plan(int m, int n, int K, int M, int nsplit, int* out6) {
   return HTR_OK;
 }
 
-void htr_set_spin_limit(int polls) { g_spin_limit = polls < 1 ? 1 : polls; }
+void htr_set_spin_limit(int polls) { g_spin_limit.store(polls < 1 ? 1 : polls, std::memory_order_relaxed); }
+
+int htr_plan_device_override(int compute_units, long lds_bytes_per_cu) {
+  if (compute_units == 0) { g_override_cus.store(0, std::memory_order_release); return HTR_OK; }
+  if (compute_units < 1 || compute_units > 4096 || lds_bytes_per_cu < 64 * 1024 || lds_bytes_per_cu > (1 << 20)) return HTR_ERR_SHAPE;
+  g_override_lds.store(lds_bytes_per_cu, std::memory_order_release);
+  g_override_cus.store(compute_units, std::memory_order_release);
+  return HTR_OK;
+}
 
 int htr_workspace_init(void* workspace, size_t workspace_bytes, void* host_status_word, void* stream) {
   if (!workspace) return HTR_ERR_NULL;
@@ -2307,7 +2352,7 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
     t.sc_g = (const float*)(wsp + align256((size_t)M * n * 2) + align256((size_t)M * (n / 128) * 16));
     t.status = (uint32_t*)workspace;
     t.cbscale = htr_cbscale();
-    t.spin_limit = g_spin_limit;
+    t.spin_limit = g_spin_limit.load(std::memory_order_relaxed);
     t.chunk_magic = 0;
     t.group = nullptr; t.group_prerot_stride = 0; t.group_part_stride = 0;
     hipStream_t st = (hipStream_t)stream;
@@ -2316,7 +2361,7 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
     if (!rot) HTR_CHECK_HIP(launch_rotation(x, (const uint8_t*)su, n, M, x_dtype, t, st));
     BatchArgs ba;
     ba.qw = (const uint32_t*)qweight; ba.part = (float*)((unsigned char*)workspace + WS_HEADER); ba.x = x; ba.su = (const uint8_t*)su;
-    ba.m = m; ba.n = n; ba.M = M; ba.flags = x_dtype | (y_dtype << 2);
+    ba.m = m; ba.n = n; ba.M = M; ba.flags = x_dtype | (y_dtype << 2) | (bp.last_finishes ? FLAG_LAST_FINISHES : 0);
     if (bp.rot && !rot) bp.lds = batch_lds_bytes(M);            // the staged kernel's layout
     HTR_FOR_K(K, return launch_batch_k<KK>(ba, rot, t, bp, st));
     return HTR_OK;
@@ -2350,7 +2395,7 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
   t.xt_g = nullptr; t.xs_g = nullptr; t.sc_g = nullptr;
   t.status = (uint32_t*)workspace;
   t.cbscale = htr_cbscale();
-  t.spin_limit = g_spin_limit;
+  t.spin_limit = g_spin_limit.load(std::memory_order_relaxed);
   t.group = nullptr; t.group_prerot_stride = 0; t.group_part_stride = 0;
   t.chunk_magic = (((unsigned long long)1 << 40) + (unsigned)pl.chunk - 1) / (unsigned)pl.chunk;
   hipStream_t st = (hipStream_t)stream;
@@ -2370,7 +2415,6 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
 static __device__ __align__(256) unsigned char scratch[HTR_STATIC_SCRATCH_BYTES];
 
 namespace {
-constexpr int MAX_DEVICES = 64;
 void* g_scratch_ptr[MAX_DEVICES];                 // per device: address of `scratch` there, once looked up
 std::atomic<uint64_t> g_scratch_known{0};         // bit d: g_scratch_ptr[d] is valid
 }
@@ -2409,7 +2453,7 @@ static bool make_group_plan(int count, int m, int n, int max_M, Plan& pl) {
   // aim at a few workgroups per CU over all problems; chunks are whole rows of column blocks or divide one, so that
   // no chunk straddles a row block; of those the one nearest the target (in ratio) that fits LDS
   static const int per_cu = getenv("HTR_GROUP_WGS_PER_CU") ? atoi(getenv("HTR_GROUP_WGS_PER_CU")) : 4;
-  const double target = (double)vtotal * count / ((double)(per_cu > 0 ? per_cu : 4) * NUM_CU);
+  const double target = (double)vtotal * count / ((double)(per_cu > 0 ? per_cu : 4) * num_cu());
   double best = 1e30;
   bool found = false;
   for (long chunk = 1; chunk <= vtotal && chunk <= MAX_CHUNK; ++chunk) {
@@ -2459,7 +2503,7 @@ int htr_linear_grouped(const htr_group_entry* entries, int count, int m, int n, 
   t.sc_g = (const float*)(wsp + align256((size_t)max_M * n * 2) + align256((size_t)max_M * (n / 128) * 16));
   t.status = (uint32_t*)workspace;
   t.cbscale = htr_cbscale();
-  t.spin_limit = g_spin_limit;
+  t.spin_limit = g_spin_limit.load(std::memory_order_relaxed);
   t.chunk_magic = (((unsigned long long)1 << 40) + (unsigned)pl.chunk - 1) / (unsigned)pl.chunk;
   t.group = entries; t.group_prerot_stride = pre; t.group_part_stride = (unsigned long long)pl.wgs * max_M * 128;
   hipStream_t st = (hipStream_t)stream;

@@ -103,14 +103,27 @@ unsigned long long htr_stream_capture_id(void* stream);
  * workgroup, 1 if the activations are rotated by a launch of their own, dynamic LDS bytes}.  No reference counterpart
  * as a function; it exposes what nsplit_for / fused_nsplit decide there (htr/ops.py:31-45).
  * With 9 rows and more (6 and more for m >= 24576, 7 and more where a full grid has splits of at most four column blocks;
- * library policy) the batched kernel runs instead: out6 = {column blocks per split, workgroups
- * (= row blocks x splits), 1, 1, 1 if the activations are rotated by a launch of their own (0: up to 16 rows over at most 16 column
- * blocks per split, where the workgroups rotate their own slices), dynamic LDS bytes}.
+ * library policy) the batched kernel runs instead: out6 = {column blocks per split, workgroups (= row blocks x splits),
+ * 1 if the splits of a row block finish rows for each other (only while the grid is at most one workgroup per compute
+ * unit; 0: the last split finishes every row), splits per row block, 1 if the activations are rotated by a launch of their
+ * own (0: the workgroups rotate their own slices: up to 16 rows over at most 16 column blocks per split, or up to 32 rows
+ * over at most 8), dynamic LDS bytes}.  Entries 4 and 5 assume bf16 / f16 activations on a 16-byte boundary; float32 or
+ * otherwise aligned activations always take the rotation launch and the staged kernel's LDS layout.
+ * Plans are made for the current device's compute-unit count and LDS size (an unpartitioned MI355X where no device can
+ * be asked); see htr_plan_device_override.
  * nsplit: 0 = library policy; otherwise the steps per workgroup of the chunked kernel (1 .. HTR_MAX_GROUP_ROWS rows;
  * bit 30 set: force the separate rotation launch), or, with bit 29 set, the batched kernel with that many column
  * splits in the low bits (0 = its own policy).
  */
 int htr_linear_plan(int m, int n, int K, int M, int nsplit, int* out6);
+
+/*
+ * Makes every later plan assume a device of `compute_units` compute units with `lds_bytes_per_cu` bytes of LDS each,
+ * instead of what the runtime reports for the current device; compute_units = 0 returns to the device's own figures.
+ * For tests of the planner and for tuning; the kernels themselves are correct for any plan the library hands out.
+ * Reference: the environment override of the workgroup target, HTR_FUSED_WGS (htr/ops.py:44).
+ */
+int htr_plan_device_override(int compute_units, long lds_bytes_per_cu);
 
 /*
  * y[M, m] = x[M, n] @ W^T (+ bias) for an HTR-W1 weight, one fused launch: input sign flip +

@@ -614,3 +614,33 @@ def test_batched_kernel_with_explicit_splits(dev, oracle, M, S, monkeypatch):
     monkeypatch.setattr(ops, "NSPLIT", (1 << 29) | S)
     y = ops.linear_f32out(x.to(dev), *[t.to(dev) for t in (qw, sc, su, sv)]).cpu().numpy()
     assert _rel(y, _ref(oracle, qw, sc, su, sv, x)) <= REL_TOL
+
+
+@pytest.mark.parametrize("M,S", [(12, 4), (24, 4), (32, 8), (64, 2), (100, 4), (128, 8)])
+def test_batched_kernel_when_the_grid_exceeds_the_compute_units(dev, oracle, M, S, monkeypatch):
+    """With a device of fewer compute units than the grid has workgroups (forced through the planner's override), the
+    splits of a row block may not wait for each other: the last split finishes every row.  Same results, and with the
+    override lifted the same explicit plan goes back to the splits sharing the output side."""
+    import ctypes
+    from htr_amd import _native, ops
+    print(f"batched kernel, grid beyond the CU count M={M} S={S}", flush=True)
+    L = _native.lib()
+    m, n = 1024, 2048
+    qw, sc, su, sv, x = _case(m, n, 4, M, 6100 + 10 * M + S)
+    d = [t.to(dev) for t in (qw, sc, su, sv)]
+    ref = _ref(oracle, qw, sc, su, sv, x)
+    out = (ctypes.c_int * 6)()
+    monkeypatch.setattr(ops, "NSPLIT", (1 << 29) | S)
+    assert L.htr_plan_device_override(8, 160 * 1024) == 0
+    try:
+        assert L.htr_linear_plan(m, n, 4, M, (1 << 29) | S, out) == 0 and out[1] == 8 * S and out[2] == 0
+        ops._NEED.clear()
+        y_small = ops.linear_f32out(x.to(dev), *d).cpu().numpy()
+    finally:
+        assert L.htr_plan_device_override(0, 0) == 0
+        ops._NEED.clear()
+    assert L.htr_linear_plan(m, n, 4, M, (1 << 29) | S, out) == 0 and out[2] == 1
+    y_full = ops.linear_f32out(x.to(dev), *d).cpu().numpy()
+    assert _rel(y_small, ref) <= REL_TOL and _rel(y_full, ref) <= REL_TOL
+    # the sums run over the same partials in the same order either way
+    assert np.abs(y_small - y_full).max() <= 2e-6 * np.abs(ref).max()

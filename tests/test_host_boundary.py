@@ -108,6 +108,44 @@ def test_launch_plan_is_consistent(L, m, n, M):
         assert out[1] == rbs * nblk
 
 
+@pytest.mark.parametrize("cus", [32, 64, 120, 256, 304])
+def test_plans_follow_the_device_compute_unit_count(L, cus):
+    """The planner with another device's compute-unit count: the batched kernel's splits may only finish rows for each
+    other (and so wait for each other) while the whole grid fits the chip at once; an explicit split beyond that falls
+    back to the last split finishing every row.  The chunked kernel's waits only look at earlier workgroups, so any grid
+    is safe there; its plan must still tile the step space."""
+    out = (ctypes.c_int * 6)()
+    assert L.htr_plan_device_override(cus, 160 * 1024) == 0
+    try:
+        for m, n in [(1024, 4096), (4096, 4096), (14336, 4096), (4096, 14336), (28672, 4096)]:
+            nblk, rbs = n // 128, m // 128
+            for M in (9, 16, 17, 32, 64, 128):
+                assert L.htr_linear_plan(m, n, 4, M, 0, out) == 0
+                cb, wgs, mutual, S, prerot, lds = list(out)
+                assert wgs == rbs * S and S == -(-nblk // cb)
+                assert wgs <= cus or S == 1                            # the policy never oversubscribes with splits
+                assert mutual == (1 if wgs <= cus else 0)
+                if prerot == 0:
+                    assert wgs <= cus                                  # workgroups rotate their own slices only on a grid that fits
+                for want in (2, 4, 8):
+                    if L.htr_linear_plan(m, n, 4, M, (1 << 29) | want, out) != 0:
+                        continue
+                    assert out[3] == want and out[1] == rbs * want
+                    assert out[2] == (1 if rbs * want <= cus else 0)   # mutual waits only when every workgroup is resident
+                    assert L.htr_workspace_bytes(m, n, 4, M, (1 << 29) | want) >= 256 + out[1] * M * 128 * 4
+            for M in (1, 4, 8):
+                assert L.htr_linear_plan(m, n, 4, M, 0, out) == 0
+                if M < 6 or (M < 7 and rbs < 192):
+                    chunk, wgs = out[0], out[1]
+                    assert (wgs - 1) * chunk < rbs * nblk <= wgs * chunk
+        assert L.htr_plan_device_override(-1, 160 * 1024) == 3 and L.htr_plan_device_override(64, 1024) == 3
+    finally:
+        assert L.htr_plan_device_override(0, 0) == 0
+    # back on the default device (none here: an unpartitioned MI355X is assumed): the decoder layer's batch-1 plans fill it
+    for m, n in [(6144, 4096), (4096, 4096), (28672, 4096), (4096, 14336)]:
+        assert L.htr_linear_plan(m, n, 4, 1, 0, out) == 0 and out[1] == 256
+
+
 def test_wire_helpers_match_oracle(oracle):
     from htr_amd import wire
     signs = torch.tensor([1., -1., 1., -1., 1., -1., 1., -1.])

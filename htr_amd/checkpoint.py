@@ -176,8 +176,10 @@ def write_packed_chunk(path, L, K, experts, extra=None):
 def read_packed_chunk(path, device="cpu", verify=False):
     """One chunk file -> {"L", "K", "experts": {e: {"n", "gate", "up", "down", "what_bf16_sha256"}}} with every role an
     HTR-W1 tuple (qweight, scales, su, sv) on `device`.  The file is unpickled with torch's weights-only loader: tensors,
-    numbers, strings, lists and dicts, nothing that runs code.  verify=True also recomputes the reconstruction hashes
-    (decodes every matrix on the host: slow for real experts)."""
+    numbers, strings, lists and dicts, nothing that runs code.  Shapes, K and the MLP structure are always checked; the
+    encoder's reconstruction hashes (what_bf16_sha256) are NOT, unless asked for: verify=True recomputes all of them
+    (decodes every matrix on the host with torch: about a second per real expert matrix), verify="first" only those of
+    the chunk's first expert (a cheap guard against a chunk written with another codebook or bit order)."""
     z = torch.load(path, map_location="cpu", weights_only=True)
     if not isinstance(z, dict) or z.get("format") != PACKED_FORMAT:
         raise ValueError(f"{path}: not a {PACKED_FORMAT} chunk (format = {z.get('format') if isinstance(z, dict) else type(z).__name__!r})")
@@ -185,7 +187,7 @@ def read_packed_chunk(path, device="cpu", verify=False):
     if not 2 <= K <= 8:
         raise ValueError(f"{path}: K = {K} outside 2..8")
     experts = {}
-    for ex in z["experts"]:
+    for pos, ex in enumerate(z["experts"]):
         e = int(ex["e"])
         if e in experts:
             raise ValueError(f"{path}: expert {e} appears twice")
@@ -196,7 +198,7 @@ def read_packed_chunk(path, device="cpu", verify=False):
             m, n, k = wire.check_shapes(*t)
             if k != K:
                 raise ValueError(f"{path}: expert {e} {role} has K = {k}, the chunk says {K}")
-            if verify:
+            if verify is True or (verify == "first" and pos == 0):
                 import hashlib
                 got = hashlib.sha256(wire.dequant(*t).bfloat16().contiguous().view(torch.int16).numpy().tobytes()).hexdigest()
                 want = rec["what_bf16_sha256"].get(role)
@@ -246,7 +248,9 @@ class PackedExperts:
 
     def layer(self, L, device="cpu", verify=False):
         """(gate_up, down, K): lists indexed by expert id, ready for ops.moe_experts.  Raises if the layer's chunks leave
-        a hole in the expert ids, disagree in K, or name another layer."""
+        a hole in the expert ids, disagree in K, or name another layer.  The reconstruction hashes in the chunks go
+        unchecked by default; verify="first" checks the first expert of every chunk, verify=True all of them (see
+        read_packed_chunk for the cost)."""
         recs, K = {}, None
         for p in self.chunks(L):
             z = read_packed_chunk(p, device, verify)

@@ -41,23 +41,52 @@ class _Workspace:
         self.buf, self.flag, self.stream = buf, flag, stream
 
 
-_WORKSPACES = {}      # (device index, stream) or (device index, "capture", capture id) -> _Workspace
-_RETIRED = []         # buffers that a capture in progress has already recorded launches with: never freed
-_FLAG_POOLS = {}      # device index -> [pinned int32 tensor, its numpy view, next free word]
+_WORKSPACES = {}      # (device index, stream), (device index, "capture", capture id) or (device index, "shared") -> _Workspace
+_RETIRED = []         # buffers that a capture in progress has already recorded launches with: kept until released
+_FLAG_POOLS = {}      # device index -> list of [pinned int32 tensor, its numpy view, next free word]
 _FLAG_WORDS = 1024
+# Captures that replay one after the other on one stream (the piecewise graphs of a serving stack: one per layer and batch
+# size, thousands of them) may share ONE workspace per device instead of each holding its own: set this (or
+# HTR_SHARE_CAPTURE_WS=1) before capturing.  Graphs that share it must never replay concurrently.
+SHARE_CAPTURE_WORKSPACE = os.environ.get("HTR_SHARE_CAPTURE_WS", "0") not in ("", "0")
+
+
+def share_capture_workspace(on=True):
+    """Opt in to (or out of) one shared workspace per device for all HIP-graph captures: it is allocated and zeroed once,
+    outside any capture (a warm-up call, or reserve_capture_workspace), so a capture neither allocates nor records a fill
+    kernel, and thousands of captured pieces cost one buffer.  Only for graphs that replay serially."""
+    global SHARE_CAPTURE_WORKSPACE
+    SHARE_CAPTURE_WORKSPACE = bool(on)
+
+
+def reserve_capture_workspace(device, nbytes):
+    """Allocates (outside a capture) the shared capture workspace of `device` with room for `nbytes`."""
+    device = torch.device(device)
+    if torch.cuda.is_current_stream_capturing():
+        raise RuntimeError("reserve_capture_workspace must be called outside a capture")
+    with torch.cuda.device(device):
+        return _shared_workspace(device, _raw_stream(device.index), int(nbytes))
+
+
+def release_capture_workspaces(device=None):
+    """Drops the workspaces that captures on `device` (all devices if None) own.  Call it only after the graphs that
+    recorded them have been destroyed: a graph replayed afterwards would write into freed memory."""
+    dev = None if device is None else torch.device(device).index
+    for key in [k for k in _WORKSPACES if len(k) == 3 and (dev is None or k[0] == dev)]:
+        del _WORKSPACES[key]
+    _RETIRED[:] = [w for w in _RETIRED if dev is not None and w.buf.device.index != dev]
 
 
 def _flag_word(device):
-    """A 4-byte word of pinned host memory (None while a capture is in progress and no pool exists yet, or when the
-    pool is used up: the workspace then works without a host-side flag)."""
-    pool = _FLAG_POOLS.get(device.index)
-    if pool is None:
+    """A 4-byte word of pinned host memory (None while a capture is in progress and no room is left in the pools
+    allocated so far: that workspace then works without a host-side flag)."""
+    pools = _FLAG_POOLS.setdefault(device.index, [])
+    if not pools or pools[-1][2] >= _FLAG_WORDS:
         if torch.cuda.is_current_stream_capturing():
             return None
         t = torch.zeros(_FLAG_WORDS, dtype=torch.int32).pin_memory()
-        pool = _FLAG_POOLS[device.index] = [t, t.numpy(), 0]
-    if pool[2] >= _FLAG_WORDS:
-        return None
+        pools.append([t, t.numpy(), 0])
+    pool = pools[-1]
     i = pool[2]
     pool[2] += 1
     return pool[1][i:i + 1], pool[0].data_ptr() + 4 * i
@@ -81,18 +110,49 @@ def check_status(device=None):
             _heal(ws, torch.device("cuda", key[0]))
 
 
+def _new_workspace(key, device, stream_id, size):
+    buf = torch.empty(size, dtype=torch.uint8, device=device)
+    flag = _flag_word(device)
+    ws = _WORKSPACES[key] = _Workspace(buf, flag, stream_id)
+    _native.check(_native.lib().htr_workspace_init(buf.data_ptr(), size, None if flag is None else flag[1], stream_id))
+    return ws
+
+
+def _shared_workspace(device, stream_id, nbytes):
+    key = (device.index, "shared")
+    ws = _WORKSPACES.get(key)
+    if ws is not None and ws.buf.numel() >= nbytes:
+        return ws.buf
+    if torch.cuda.is_current_stream_capturing():
+        raise RuntimeError(f"libhtr_gfx950: the shared capture workspace of {device} holds "
+                           f"{0 if ws is None else ws.buf.numel()} bytes, this launch needs {nbytes}; run the shapes once outside "
+                           "the capture first, or call ops.reserve_capture_workspace")
+    if ws is not None:
+        _RETIRED.append(ws)        # graphs captured so far keep replaying against the old buffer
+    return _new_workspace(key, device, stream_id, max(int(nbytes), 1 << 20)).buf
+
+
 def workspace(device, stream_id, nbytes):
     """Scratch for split partials and pre-rotated activations: one per (device, stream), and one per HIP-graph capture.
 
     The reference keeps one counter tensor per device (htr/ops.py:24-28), which two streams
     would corrupt; keying by stream keeps concurrent streams apart.  Kernels leave the
     partial slots zero, so a buffer is cleared only when it is created (by the library's fill kernel).
-    Every capture gets buffers of its own (keyed by the runtime's capture id), allocated inside the capture, i.e. from
-    the graph's memory pool, and kept alive here for good: its address is part of the recorded launches.  A buffer
-    that a capture has used is never replaced or freed; if a later call of the same capture needs more, a further
-    buffer is added.  Eager calls never touch a capture's buffers.
+    By default every capture gets buffers of its own (keyed by the runtime's capture id), allocated inside the capture,
+    i.e. from the graph's memory pool, sized to what its launches need (no floor: a batch-1 layer takes tens of KB), and
+    kept alive here until release_capture_workspaces: its address is part of the recorded launches, and the fill kernel
+    of a NEW buffer is recorded with them.  A buffer that a capture has used is never replaced or freed; if a later call
+    of the same capture needs more, a further buffer is added.  Eager calls never touch a capture's buffers.
+    With SHARE_CAPTURE_WORKSPACE all captures of a device use one buffer that exists before they start (no allocation
+    and no fill in any capture); that is only right for graphs that replay one after the other.
     """
-    cid = _native.lib().htr_stream_capture_id(stream_id) if torch.cuda.is_current_stream_capturing() else 0
+    capturing = torch.cuda.is_current_stream_capturing()
+    if capturing and SHARE_CAPTURE_WORKSPACE:
+        return _shared_workspace(device, stream_id, nbytes)
+    if not capturing and SHARE_CAPTURE_WORKSPACE:
+        # eager calls (the warm-up before the captures) size the shared buffer; they run on their own stream's buffer
+        _shared_workspace(device, stream_id, nbytes)
+    cid = _native.lib().htr_stream_capture_id(stream_id) if capturing else 0
     key = (device.index, "capture", cid) if cid else (device.index, stream_id)
     ws = _WORKSPACES.get(key)
     if ws is not None and ws.buf.numel() >= nbytes:
@@ -101,12 +161,8 @@ def workspace(device, stream_id, nbytes):
         return ws.buf
     if ws is not None and cid:
         _RETIRED.append(ws)
-    size = max(int(nbytes), 1 << 20)
-    buf = torch.empty(size, dtype=torch.uint8, device=device)
-    flag = _flag_word(device)
-    ws = _WORKSPACES[key] = _Workspace(buf, flag, stream_id)
-    _native.check(_native.lib().htr_workspace_init(buf.data_ptr(), size, None if flag is None else flag[1], stream_id))
-    return buf
+    size = (int(nbytes) + 255) // 256 * 256 if cid else max(int(nbytes), 1 << 20)
+    return _new_workspace(key, device, stream_id, size).buf
 
 
 _NEED = {}       # workspace bytes per (m, n, K, M, nsplit)

@@ -123,6 +123,15 @@ def test_packed_chunk_round_trip_and_refusals(tmp_path):
     checkpoint.read_packed_chunk(str(root / "L0" / "c000.pt"))
     with pytest.raises(ValueError, match="reconstruction hash"):
         checkpoint.read_packed_chunk(str(root / "L0" / "c000.pt"), verify=True)
+    with pytest.raises(ValueError, match="reconstruction hash"):
+        checkpoint.read_packed_chunk(str(root / "L0" / "c000.pt"), verify="first")     # the flipped bit is in the first expert
+    z2 = torch.load(str(root / "L0" / "c000.pt"), weights_only=True)
+    z2["experts"][0]["packed"]["down"]["qweight"][0, 0, 0] ^= 1                        # first expert whole again,
+    z2["experts"][1]["packed"]["up"]["qweight"][0, 0, 0] ^= 1                          # the second one damaged
+    torch.save(z2, str(tmp_path / "second.pt"))
+    checkpoint.read_packed_chunk(str(tmp_path / "second.pt"), verify="first")          # the cheap check looks at the first only
+    with pytest.raises(ValueError, match="reconstruction hash"):
+        checkpoint.read_packed_chunk(str(tmp_path / "second.pt"), verify=True)
     # another format string, a hole in the expert ids, gate/up with different su, mixed K in one layer, wrong layer
     z["format"] = "HTR-W1-P1"
     torch.save(z, str(tmp_path / "bad.pt"))

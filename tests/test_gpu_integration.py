@@ -277,6 +277,67 @@ def test_captures_own_their_workspaces(dev):
     del filler
 
 
+def test_captures_can_share_one_workspace(dev):
+    """Opt-in for serving stacks that capture thousands of pieces which replay one after the other: all captures of a
+    device use one workspace that exists before they start, so a capture allocates nothing and records no fill kernel.
+    A capture that would need more than the shared buffer holds is refused with a clear error (inside the capture
+    nothing may be allocated), and a capture's own workspace, in the default mode, is sized to the launch, not to 1 MiB."""
+    from htr_amd import ops, wire
+    print("shared capture workspace", flush=True)
+    qw, sc, su, sv, x = _case(1024, 2048, 4, 1, 4800)
+    d = [t.to(dev) for t in (qw, sc, su, sv)]
+    d2 = [t.to(dev) for t in wire.synth_linear(2048, 1024, 3, 4801)]
+    x1, x2 = x.to(dev).clone(), wire.synth_activation(3, 1024, 4802).to(dev)
+    want1, want2 = ops.linear(x1, *d), ops.linear(x2, *d2)
+    torch.cuda.synchronize()
+    # default mode: one buffer per capture, as large as the launch needs
+    g0 = torch.cuda.CUDAGraph()
+    before = set(ops._WORKSPACES)
+    with torch.cuda.graph(g0):
+        y0 = ops.linear(x1, *d)
+    own = [ops._WORKSPACES[k] for k in set(ops._WORKSPACES) - before]
+    assert len(own) == 1 and own[0].buf.numel() < (1 << 20)
+    g0.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(y0, want1)
+    ops.share_capture_workspace(True)
+    try:
+        ops.linear(x1, *d)
+        ops.linear(x2, *d2)                      # the warm-up pass sizes the shared buffer
+        torch.cuda.synchronize()
+        shared = ops._WORKSPACES[(dev.index, "shared")]
+        before = set(ops._WORKSPACES)
+        g1, g2 = torch.cuda.CUDAGraph(), torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g1):
+            y1 = ops.linear(x1, *d)
+        with torch.cuda.graph(g2):
+            y2 = ops.linear(x2, *d2)
+        assert set(ops._WORKSPACES) == before and ops._WORKSPACES[(dev.index, "shared")] is shared
+        for _ in range(3):
+            g1.replay()
+            g2.replay()
+            ops.linear(x2, *d2)                  # eager work between the replays
+            torch.cuda.synchronize()
+            assert torch.equal(y1, want1) and torch.equal(y2, want2)
+        big = [t.to(dev) for t in wire.synth_linear(14336, 4096, 4, 4803)]
+        xb = wire.synth_activation(100, 4096, 4804).to(dev)
+        g3 = torch.cuda.CUDAGraph()
+        with pytest.raises(RuntimeError, match="shared capture workspace"):
+            with torch.cuda.graph(g3):
+                ops.linear(xb, *big)
+        torch.cuda.synchronize()
+        ops.reserve_capture_workspace(dev, 64 << 20)
+        with torch.cuda.graph(g3):
+            y3 = ops.linear(xb, *big)
+        g3.replay()
+        g1.replay()                              # the earlier graphs still replay against the buffer they recorded
+        torch.cuda.synchronize()
+        assert torch.equal(y1, want1)
+        assert torch.equal(y3, ops.linear(xb, *big))
+    finally:
+        ops.share_capture_workspace(False)
+
+
 def test_packed_expert_chunks_feed_the_grouped_launch(dev, oracle):
     """The committed routed-expert chunks (reference layout, htr/moe_encode.py:216-225; four experts, K3) are read with
     the weights-only loader, fused to gate_up / down lists and run through ops.moe_experts; the result is compared with

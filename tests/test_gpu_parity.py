@@ -642,5 +642,5 @@ def test_batched_kernel_when_the_grid_exceeds_the_compute_units(dev, oracle, M, 
     assert L.htr_linear_plan(m, n, 4, M, (1 << 29) | S, out) == 0 and out[2] == 1
     y_full = ops.linear_f32out(x.to(dev), *d).cpu().numpy()
     assert _rel(y_small, ref) <= REL_TOL and _rel(y_full, ref) <= REL_TOL
-    # the sums run over the same partials in the same order either way
-    assert np.abs(y_small - y_full).max() <= 2e-6 * np.abs(ref).max()
+    # the same products either way (the rotation may come from the launch of its own in one and from the workgroups in the other)
+    assert np.abs(y_small - y_full).max() <= 2e-4 * np.abs(ref).max()

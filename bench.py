@@ -45,9 +45,12 @@ def parse():
     ap.add_argument("--no-shapes", action="store_true", help="skip the per-shape table and the unfused layer")
     ap.add_argument("--viterbi-tiles", type=int, default=0,
                     help="also time the encoder's trellis search on this many 256-weight tiles per K (0 = skip)")
-    ap.add_argument("--suite", nargs="*", default=None, metavar="CASE",
-                    help="also time the other baseline configurations (bench_suite.py): table, batch, layer_rows, lm_head, moe, "
-                         "prefill; no names = all")
+    ap.add_argument("--repeats", type=int, default=7, help="timed passes of the headline graph (median and min are reported)")
+    ap.add_argument("--suite", nargs="*", default=["default"], metavar="CASE",
+                    help="the other baseline configurations (bench_suite.py): default = table (K2..5 x 2 shapes x batch 1, 2, 4), "
+                         "batch8_32 (K3, K4 x 8, 16, 32 rows x 2 shapes), moe, lm_head; further names: batch, layer_rows, prefill, "
+                         "all; none = skip")
+    ap.add_argument("--no-anchors", action="store_true", help="skip the timing anchors of the dominant kernel")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy, so a counter profile of this command holds a kernel of known traffic")
     return ap.parse_args()
@@ -181,7 +184,8 @@ def main():
     while time.perf_counter() - t_spin < 0.03:
         run_steps()
         torch.cuda.synchronize()
-    dev_us, wall_us = timed(run_steps, args.steps)
+    passes = sorted((timed(run_steps, args.steps)[::-1] for _ in range(max(1, args.repeats))))      # (wall, device) pairs
+    wall_us, dev_us = passes[len(passes) // 2]
     ms_per_step = wall_us * 1e-3
     value = layer_bytes / (ms_per_step * 1e-3) / 1e9
 
@@ -223,6 +227,47 @@ def main():
                                 "peak": round(peak, 2), "frac": round(lane_ops / dom_us / 1e6 / peak, 4),
                                 "valu_instructions_per_weight": round(cj["valu_instructions_per_launch"] * 64 / cj["weights_per_launch"], 3),
                                 "source": "instruction counts from profiles/k_linear_K4_gate_up_sq_counters.json (committed), duration from this run"}
+
+    # ---- timing anchors of the dominant launch, same ring, same run: its bytes read and nothing else; the launch with
+    # the decode compiled out; the decode loop on register data (shader clock).  They bound what the exact decode allows.
+    if not args.no_anchors:
+        def anchor_launcher(kind):
+            def go(i):
+                p = gate_up[i % len(gate_up)]
+                st = torch.cuda.current_stream().cuda_stream
+                _native.check(L.htr_anchor_linear(kind, p.qw.data_ptr(), p.sc.data_ptr(), p.su.data_ptr(), p.sv.data_ptr(),
+                                                  xs[p.n].data_ptr(), ys[p.m].data_ptr(), p.m, p.n, p.k, _native.BF16, _native.BF16,
+                                                  ws.data_ptr(), ws.numel(), st))
+            return go
+        reps = max(110, min(args.steps, 440))
+        anchors = {}
+        for name, kind in (("plain_read_us", 2), ("no_decode_us", 1)):
+            run = make_runner(anchor_launcher(kind), reps)
+            run()
+            anchors[name] = round(sorted(timed(run, reps)[0] for _ in range(3))[1], 3)
+        _native.check(L.htr_workspace_init(ws.data_ptr(), ws.numel(), None, torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
+        iters, wgs = 4000, 256
+        stamps = torch.zeros(wgs * 8 * 2, dtype=torch.int64, device=dev)
+        for name, mf in (("decode_only", 0), ("decode_and_products", 1)):
+            for _ in range(2):
+                _native.check(L.htr_anchor_decode(K, mf, iters, wgs, stamps.data_ptr(), torch.cuda.current_stream().cuda_stream))
+                torch.cuda.synchronize()
+            t = stamps.view(-1, 2).double().cpu()
+            cyc, ghz = float(t[:, 0].median()) / iters / 2.0, float((t[:, 0] / (t[:, 1] * 10.0)).median())
+            anchors[name + "_cycles_per_wave_step"] = round(cyc, 1)           # per SIMD: two waves share it
+            anchors[name + "_shader_clock_GHz"] = round(ghz, 3)
+            # all wave-steps of the launch spread over the chip's SIMDs (4 per CU) at that rate and clock
+            simds = 4 * torch.cuda.get_device_properties(dev).multi_processor_count
+            us = (gate_up[0].m // 16) * (gate_up[0].n // 128) / simds * cyc / (ghz * 1e3)
+            anchors[name + "_us"] = round(us, 3)
+        roofline["anchors"] = anchors
+        roofline["anchors_note"] = ("same ring and run as us_per_launch: plain_read_us = the launch's weight stream and nothing else; "
+                                    "no_decode_us = the launch with the trellis decode compiled out; decode_*_cycles_per_wave_step = the "
+                                    "decode (and the four matrix instructions) of 2048 weights on register data, per SIMD, two waves per "
+                                    "SIMD; *_us = all wave-steps of the launch over all SIMDs at that rate")
+        roofline["ceiling_frac"] = round(dom_bytes / anchors["decode_only_us"] / 1e3 / HBM_PEAK_GBS, 4)
+        roofline["ceiling_frac_with_products"] = round(dom_bytes / anchors["decode_and_products_us"] / 1e3 / HBM_PEAK_GBS, 4)
 
     if args.calibrate_copy:
         src = torch.randint(0, 256, (256 << 20,), dtype=torch.uint8, device=dev)
@@ -318,7 +363,7 @@ def main():
                 search[f"K{k}"]["cpu_port_tiles_per_s"] = round(nt / (time.perf_counter() - t), 1)
 
     suite = None
-    if args.suite is not None:
+    if args.suite and "none" not in args.suite:
         import bench_suite
         del layers, gate_up, unfused
         torch.cuda.empty_cache()
@@ -337,6 +382,9 @@ def main():
         "pct_hbm": round(value / HBM_PEAK_GBS * 100, 2),
         "us_per_layer": round(ms_per_step * 1e3, 2),
         "us_per_layer_device_events": round(dev_us, 2),
+        "timed_passes": {"count": len(passes), "of_steps_each": args.steps, "us_per_layer_wall_median": round(wall_us, 2),
+                         "us_per_layer_wall_min": round(passes[0][0], 2), "us_per_layer_wall_max": round(passes[-1][0], 2),
+                         "us_per_layer_device_events_min": round(min(p[1] for p in passes), 2)},
         "verified": verified,
         "roofline": roofline,
         "cpu_baseline": cpu,

@@ -101,6 +101,18 @@ def layer_rows(dev):
     return out
 
 
+def batch8_32(dev):
+    """K3, K4 x 8, 16, 32 activation rows x {14336x4096, 4096x14336}, with the rate in TFLOP/s (2 M m n)."""
+    out = []
+    for K in (3, 4):
+        for M in (8, 16, 32):
+            for (m, n) in ((14336, 4096), (4096, 14336)):
+                r = time_linear(m, n, K, M, dev)
+                r["TFLOPs"] = round(2.0 * M * m * n / r["us"] / 1e6, 1)
+                out.append(r)
+    return out
+
+
 def lm_head(dev):
     return time_linear(152064, 4096, 4, 1, dev, ring_bytes=1 << 30, launches=96)      # few launches leave the clocks unsettled
 
@@ -202,12 +214,14 @@ def prefill(dev):
     return out
 
 
-CASES = {"table": table, "batch": batch, "layer_rows": layer_rows, "lm_head": lm_head, "moe": moe, "prefill": prefill}
+CASES = {"table": table, "batch8_32": batch8_32, "moe": moe, "lm_head": lm_head, "batch": batch, "layer_rows": layer_rows,
+         "prefill": prefill}
+DEFAULT = ("table", "batch8_32", "moe", "lm_head")       # what bench.py reports by default: every baseline configuration
 
 
 def run(names, dev=None):
     dev = dev or torch.device("cuda:0")
-    names = list(CASES) if not names or "all" in names else names
+    names = list(CASES) if not names or "all" in names else [c for nm in names for c in (DEFAULT if nm == "default" else (nm,))]
     res = {}
     for nm in names:
         res[nm] = CASES[nm](dev)

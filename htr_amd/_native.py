@@ -31,6 +31,8 @@ SIGNATURES = {
     "htr_plan_device_override": (_i, [_i, ctypes.c_long]),
     "htr_linear": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
     "htr_linear_static": (_i, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp]),
+    "htr_anchor_linear": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
+    "htr_anchor_decode": (_i, [_i, _i, _i, _i, _vp, _vp]),
     "htr_grouped_workspace_bytes": (_sz, [_i, _i, _i, _i, _i]),
     "htr_linear_grouped": (_i, [_vp, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp]),
     "htr_set_spin_limit": (None, [_i]),

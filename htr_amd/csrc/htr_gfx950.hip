@@ -542,7 +542,14 @@ __global__ __launch_bounds__(WG_THREADS) void k_rotate_mfma(const void* __restri
 
 template <int K> struct DecodedStep { h8 a[4]; };   // MFMA A operands of one step: (row 2q | 2q+1) x (columns 0..7 | 8..15)
 
-template <int K> __device__ __forceinline__ void decode_step(const StreamRegs<K>& r, int hist, DecodedStep<K>& d) {
+// NODECODE (timing anchors only): the operands are the raw stream words, no arithmetic at all; results are meaningless
+template <int K, bool NODECODE = false> __device__ __forceinline__ void decode_step(const StreamRegs<K>& r, int hist, DecodedStep<K>& d) {
+  if constexpr (NODECODE) {
+    const u4 raw = {r.d[0], r.d[1 % K], r.d[2 % K], r.d[3 % K]};
+#pragma unroll
+    for (int k = 0; k < 4; ++k) d.a[k] = __builtin_bit_cast(h8, raw);
+    return;
+  }
   // The history dword travels through the LDS crossbar.  Only the first states of the lane reach into it, so their
   // group is decoded last, behind a scheduling fence: the crossbar latency hides behind the other three groups.
   const uint32_t prev = (uint32_t)__builtin_amdgcn_ds_bpermute(hist, (int)r.d[K - 1]);
@@ -595,7 +602,9 @@ constexpr int FLAG_LANES = 1 << 4;     // kernel flag: chunk ids are dealt to th
 constexpr int FLAG_LAST_FINISHES = 1 << 5;   // batched kernel: the last split of a row block finishes all of its rows (see there)
 constexpr int FLAG_LANE_LEN_SHIFT = 8; // with FLAG_LANES: grid / 8 in the bits from here up (no read of the hidden grid-size argument)
 
-template <int K, int MB, int P, int D, bool PREROT, int RP>
+// ANCHOR = 1 is the same kernel with the decode compiled out (stream, rotation, products, hand-over and output side stay;
+// the results are meaningless): a timing anchor that tells how much of a launch is the decode.
+template <int K, int MB, int P, int D, bool PREROT, int RP, int ANCHOR = 0>
 __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restrict__ qw_a, const void* __restrict__ x_a,
                                                        const uint8_t* __restrict__ su_a, float* __restrict__ part_a,
                                                        int m, int n, int M_a, int chunk, int flags,
@@ -828,7 +837,7 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
   DecodedStep<K> pre[D];
 #pragma unroll
   for (int i = 0; i < D; ++i) {
-    if (i == 0 || i < nsteps) decode_step<K>(buf[i], hist, pre[i]);
+    if (i == 0 || i < nsteps) decode_step<K, ANCHOR == 1>(buf[i], hist, pre[i]);
     prefetch(buf[i]);
   }
   // The decoded operands are first used behind the barrier, in conditional code, and the compiler would sink the
@@ -1007,7 +1016,7 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
     for (int pp = 0; pp < P; ++pp) {
       StreamRegs<K>& nxt = buf[(pp + D) % P];
       consume(cur, false);
-      decode_step<K>(nxt, hist, cur);
+      decode_step<K, ANCHOR == 1>(nxt, hist, cur);
       prefetch(nxt);
     }
   }
@@ -1015,7 +1024,7 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
   for (int pp = 0; pp < P; ++pp) {
     if (v + pp < nsteps) {
       consume(cur, true);
-      if (v + pp + 1 < nsteps) decode_step<K>(buf[(pp + D) % P], hist, cur);
+      if (v + pp + 1 < nsteps) decode_step<K, ANCHOR == 1>(buf[(pp + D) % P], hist, cur);
     }
   }
 
@@ -1907,6 +1916,94 @@ __global__ __launch_bounds__(VitCfg<K>::THREADS) void k_viterbi(const float* __r
   }
 }
 
+// ------------------------------------------------------------------------------------------------ timing anchors
+// Measurement only: what a launch would cost if it did nothing but read its bytes, and what the decode costs on
+// register data.  Neither produces results.
+
+// The weight stream of k_linear and nothing else: same chunks, same descriptors, same order and depth of loads; every
+// loaded word is folded into one register so that the loads cannot be dropped.
+template <int K, int P>
+__global__ __launch_bounds__(WG_THREADS) void k_anchor_read(const uint32_t* __restrict__ qw, int m, int n, int chunk, int flags,
+                                                            unsigned long long nblk_magic, uint32_t* __restrict__ sink) {
+  const int lane = threadIdx.x & 63;
+  const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int nblk = n >> 7, vtotal = (m >> 7) * nblk;
+  int cid = (int)blockIdx.x;
+  if (flags & FLAG_LANES) cid = ((int)blockIdx.x & 7) * (flags >> FLAG_LANE_LEN_SHIFT) + ((int)blockIdx.x >> 3);
+  const int v0 = cid * chunk, nsteps = min(vtotal, v0 + chunk) - v0;
+  auto div_nblk = [&](int v) { return (int)(((unsigned long long)(unsigned)v * nblk_magic) >> 40); };
+  const int rb_first = div_nblk(v0), c0 = v0 - rb_first * nblk;
+  const int last_wraps = div_nblk(c0 + nsteps - 1);
+  constexpr int STEP_BYTES = 256 * K;
+  const uint32_t strip_bytes = (uint32_t)nblk * STEP_BYTES;
+  const uint32_t* wave_base = qw + ((size_t)(rb_first * 8 + w) * nblk + (size_t)c0) * (STEP_BYTES / 4);
+  const uint32_t extent = (uint32_t)nsteps * STEP_BYTES + (uint32_t)last_wraps * 7u * strip_bytes;
+  const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)wave_base, 0, (int)extent, 0x00020000);
+  int pf_off = lane * 4 * K, pf_blk = c0;
+  StreamRegs<K> buf[P];
+  auto prefetch = [&](StreamRegs<K>& dst) {
+    HTR_PIN();
+    load_stream_buffer<K>(rsrc, pf_off, dst);
+    pf_off += STEP_BYTES;
+    if (++pf_blk == nblk) { pf_blk = 0; pf_off += 7 * (int)strip_bytes; }
+    HTR_PIN();
+  };
+#pragma unroll
+  for (int p = 0; p < P; ++p) prefetch(buf[p]);
+  uint32_t acc = 0u;
+  for (int v = 0; v < nsteps; v += P) {
+#pragma unroll
+    for (int pp = 0; pp < P; ++pp) {
+#pragma unroll
+      for (int k = 0; k < K; ++k) acc ^= buf[pp].d[k];
+      prefetch(buf[pp]);
+    }
+  }
+  if (acc == 0x9E3779B9u && sink != nullptr) sink[0] = acc;      // practically never: keeps the loads alive
+}
+
+// The decode of k_linear's inner loop on register data, `iters` wave-steps per wave, timed with the shader clock
+// (s_memtime) and the 100 MHz reference clock (s_memrealtime) around the loop.  WITH_MFMA adds the four matrix
+// instructions of a step (constant B operands).  out[wave] = {shader cycles, reference ticks}.
+template <int K, bool WITH_MFMA>
+__global__ __launch_bounds__(WG_THREADS) void k_anchor_decode(int iters, unsigned long long* __restrict__ out, float* __restrict__ sink) {
+  const int lane = threadIdx.x & 63;      // (the launch requests dynamic LDS it never touches: one workgroup per compute unit)
+  const int hist = history_lane_byteaddr(lane);
+  StreamRegs<K> r;
+#pragma unroll
+  for (int k = 0; k < K; ++k) r.d[k] = (uint32_t)(threadIdx.x * 2654435761u) ^ (uint32_t)(k * 40503u + blockIdx.x);
+  h8 b0, b1;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) { b0[i] = (_Float16)(0.25f + (float)((lane + i) & 3)); b1[i] = (_Float16)(0.5f - (float)((lane ^ i) & 1)); }
+  f4 acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = {0.f, 0.f, 0.f, 0.f};
+  DecodedStep<K> d;
+  __syncthreads();
+  const unsigned long long c0 = __builtin_amdgcn_s_memtime(), t0 = __builtin_amdgcn_s_memrealtime();
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int k = 0; k < K; ++k) asm volatile("" : "+v"(r.d[k]));          // opaque: the decode cannot be hoisted out of the loop
+    decode_step<K>(r, hist, d);
+    if constexpr (WITH_MFMA) {
+      acc0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[0], b0, acc0, 0, 0, 0);
+      acc1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[2], b0, acc1, 0, 0, 0);
+      acc0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[1], b1, acc0, 0, 0, 0);
+      acc1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(d.a[3], b1, acc1, 0, 0, 0);
+    } else {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) asm volatile("" : : "v"(d.a[k]));         // used: the decode cannot be dropped
+    }
+  }
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  if constexpr (WITH_MFMA) { asm volatile("" : "+v"(acc0)); asm volatile("" : "+v"(acc1)); }
+  const unsigned long long c1 = __builtin_amdgcn_s_memtime(), t1 = __builtin_amdgcn_s_memrealtime();
+  if (lane == 0) {
+    const size_t wv = (size_t)blockIdx.x * WG_WAVES + (threadIdx.x >> 6);
+    out[2 * wv] = c1 - c0;
+    out[2 * wv + 1] = t1 - t0;
+  }
+  if constexpr (WITH_MFMA) { if (acc0.x + acc1.y == 12345.678f && sink != nullptr) sink[0] = acc0.x; }
+}
+
 // ------------------------------------------------------------------------------------------------ workspace set-up
 // Zeroes the first `bytes` (a multiple of 16) of a workspace and writes the header's mirror address.  A kernel, not a
 // memset, so that it can be recorded into a HIP graph.
@@ -2511,6 +2608,78 @@ int htr_linear_grouped(const htr_group_entry* entries, int count, int m, int n, 
                               (const uint8_t*)nullptr, n, x_dtype, (_Float16*)t.xt_g, (float*)t.xs_g, (float*)t.sc_g, entries,
                               (unsigned long long)pre));
   HTR_FOR_K(K, return launch_linear_k<KK>(a, true, pl.mb, pl.wgs, pl.lds, st));
+  return HTR_OK;
+}
+
+// ---- timing anchors (measurement only; see the kernels).  kind 1: htr_linear's launch for one bf16 / f16 row with the
+// decode compiled out; kind 2: only the weight stream of that launch.  Same plan, grid and LDS request as htr_linear.
+int htr_anchor_linear(int kind, const void* qweight, const void* scales, const void* su, const void* sv, const void* x, void* y,
+                      int m, int n, int K, int x_dtype, int y_dtype, void* workspace, size_t workspace_bytes, void* stream) {
+  if (!qweight || !scales || !su || !sv || !x || !y) return HTR_ERR_NULL;
+  if (K != 4 || (kind != 1 && kind != 2)) return HTR_ERR_K;
+  if (!shape_ok(m, n)) return HTR_ERR_SHAPE;
+  if (x_dtype == HTR_F32 || !dtype_ok(x_dtype) || !dtype_ok(y_dtype)) return HTR_ERR_DTYPE;
+  if (((uintptr_t)qweight & 15) || ((uintptr_t)x & 3)) return HTR_ERR_ALIGN;
+  Plan pl;
+  if (!make_plan(m, n, 1, 0, pl) || pl.prerot) return HTR_ERR_SPLIT;
+  const size_t need = htr_workspace_bytes(m, n, K, 1, 0);
+  if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255)) return HTR_ERR_WORKSPACE;
+  LinearLaunch a;
+  a.qw = (const uint32_t*)qweight; a.x = x; a.su = (const uint8_t*)su;
+  a.part = (float*)((unsigned char*)workspace + WS_HEADER);
+  a.m = m; a.n = n; a.M = 1; a.chunk = pl.chunk; a.flags = x_dtype | (y_dtype << 2); a.problems = 1;
+  const int nblk = n / 128, rbs = m / 128;
+  if (pl.chunk < nblk && nblk % pl.chunk == 0 && rbs % 8 == 0 && rbs >= 16 && pl.wgs % 8 == 0) a.flags |= FLAG_LANES | ((pl.wgs / 8) << FLAG_LANE_LEN_SHIFT);
+  a.nblk_magic = (((unsigned long long)1 << 40) + (unsigned)nblk - 1) / (unsigned)nblk;
+  LinearTail& t = a.tail;
+  t.scales = (const uint16_t*)scales; t.sv = (const uint8_t*)sv; t.bias = nullptr; t.y = y;
+  t.xt_g = nullptr; t.xs_g = nullptr; t.sc_g = nullptr;
+  t.status = (uint32_t*)workspace;
+  t.cbscale = htr_cbscale();
+  t.spin_limit = g_spin_limit.load(std::memory_order_relaxed);
+  t.group = nullptr; t.group_prerot_stride = 0; t.group_part_stride = 0;
+  t.chunk_magic = (((unsigned long long)1 << 40) + (unsigned)pl.chunk - 1) / (unsigned)pl.chunk;
+  hipStream_t st = (hipStream_t)stream;
+  const size_t lds = balanced_lds_request(pl.lds, pl.wgs);
+  if (kind == 2) {
+    HTR_CHECK_HIP(launch_kernel(k_anchor_read<4, 4>, dim3(pl.wgs), dim3(WG_THREADS), lds, st, a.qw, m, n, a.chunk, a.flags, a.nblk_magic,
+                                (uint32_t*)((unsigned char*)workspace + ws_half(workspace_bytes))));
+    return HTR_OK;
+  }
+  if (pl.chunk <= 8) {
+    HTR_CHECK_HIP((allow_full_lds<k_linear<4, 1, 4, 4, false, 1, 1>>()));
+    HTR_CHECK_HIP(launch_kernel(k_linear<4, 1, 4, 4, false, 1, 1>, dim3(pl.wgs), dim3(WG_THREADS), lds, st, a.qw, a.x, a.su, a.part,
+                                a.m, a.n, a.M, a.chunk, a.flags, a.nblk_magic, a.tail));
+  } else {
+    HTR_CHECK_HIP((allow_full_lds<k_linear<4, 1, 4, 2, false, 1, 1>>()));
+    HTR_CHECK_HIP(launch_kernel(k_linear<4, 1, 4, 2, false, 1, 1>, dim3(pl.wgs), dim3(WG_THREADS), lds, st, a.qw, a.x, a.su, a.part,
+                                a.m, a.n, a.M, a.chunk, a.flags, a.nblk_magic, a.tail));
+  }
+  return HTR_OK;
+}
+
+// The decode of one wave-step (2048 weights) on register data: `workgroups` workgroups of 8 waves, one per compute unit
+// (two waves per SIMD, as in the batch-1 launches), `iters` wave-steps each; out_u64[2 * wave] = shader-clock cycles,
+// out_u64[2 * wave + 1] = ticks of the 100 MHz reference clock over the loop.
+int htr_anchor_decode(int K, int with_mfma, int iters, int workgroups, void* out_u64, void* stream) {
+  if (!out_u64) return HTR_ERR_NULL;
+  if (K < 2 || K > 5) return HTR_ERR_K;
+  if (iters < 1 || workgroups < 1 || workgroups > 65536) return HTR_ERR_SHAPE;
+  hipStream_t st = (hipStream_t)stream;
+  const size_t lds = balanced_lds_request(1024, workgroups <= num_cu() ? num_cu() : workgroups);
+#define HTR_LAUNCH_ANCHOR(KK_, MF_)                                                                                          \
+  {                                                                                                                          \
+    HTR_CHECK_HIP((allow_full_lds<k_anchor_decode<KK_, MF_>>()));                                                            \
+    HTR_CHECK_HIP(launch_kernel(k_anchor_decode<KK_, MF_>, dim3(workgroups), dim3(WG_THREADS), lds, st, iters,               \
+                                (unsigned long long*)out_u64, (float*)nullptr));                                             \
+  }
+  switch (K) {
+    case 2: if (with_mfma) HTR_LAUNCH_ANCHOR(2, true) else HTR_LAUNCH_ANCHOR(2, false) break;
+    case 3: if (with_mfma) HTR_LAUNCH_ANCHOR(3, true) else HTR_LAUNCH_ANCHOR(3, false) break;
+    case 4: if (with_mfma) HTR_LAUNCH_ANCHOR(4, true) else HTR_LAUNCH_ANCHOR(4, false) break;
+    default: if (with_mfma) HTR_LAUNCH_ANCHOR(5, true) else HTR_LAUNCH_ANCHOR(5, false) break;
+  }
+#undef HTR_LAUNCH_ANCHOR
   return HTR_OK;
 }
 

@@ -232,6 +232,21 @@ int htr_dequant_q(const void* qweight, const void* scales, void* out_f32, int mt
 int htr_dequant_w(const void* qweight, const void* scales, const void* su, const void* sv, void* out_bf16,
                   int m, int n, int K, void* stream);
 
+/*
+ * Timing anchors: measurement only, the results they leave in y are meaningless.  No reference counterpart (the
+ * reference reports its kernel's bandwidth without such anchors, docs/METHODOLOGY.md:87-90).
+ * htr_anchor_linear: the launch htr_linear would make for ONE bf16 / f16 activation row of a K4 weight (same plan, grid
+ * and LDS request), kind 1: with the trellis decode compiled out (stream, rotation, products, hand-over and output
+ * side remain), kind 2: only the weight stream (the same descriptors, order and depth of loads, nothing else).
+ * htr_anchor_decode: the decode of the inner loop on register data (K = 2..5), `workgroups` workgroups of 8 waves,
+ * `iters` wave-steps (2048 weights each) per wave, with or without the four matrix instructions of a step;
+ * out_u64[2 w] = shader-clock cycles and out_u64[2 w + 1] = ticks of the 100 MHz reference clock wave w spent in the loop.
+ */
+int htr_anchor_linear(int kind, const void* qweight, const void* scales, const void* su, const void* sv, const void* x,
+                      void* y, int m, int n, int K, int x_dtype, int y_dtype, void* workspace, size_t workspace_bytes,
+                      void* stream);
+int htr_anchor_decode(int K, int with_mfma, int iters, int workgroups, void* out_u64, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -768,14 +768,17 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
   const uint32_t* wave_base = qw + ((size_t)(rb_first * 8 + w) * nblk + (size_t)c0) * (STEP_BYTES / 4);   // uniform
   const uint32_t extent = (uint32_t)nsteps * STEP_BYTES + (uint32_t)last_wraps * 7u * strip_bytes;
   const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)wave_base, 0, (int)extent, 0x00020000);
-  int pf_off = lane * 4 * K;         // byte offset of this lane's dwords in the next step to load
+  // the walk over the chunk's steps: a scalar byte offset (the lane adds its own), advanced without branches
+  const int lane_off = lane * 4 * K;
+  int pf_off = 0;
   int pf_blk = c0;
   StreamRegs<K> buf[P];
   auto prefetch = [&](StreamRegs<K>& dst) {
     HTR_PIN();
-    load_stream_buffer<K>(rsrc, pf_off, dst);
-    pf_off += STEP_BYTES;
-    if (++pf_blk == nblk) { pf_blk = 0; pf_off += 7 * (int)strip_bytes; }
+    load_stream_buffer<K>(rsrc, lane_off + pf_off, dst);
+    const bool wrap = pf_blk == nblk - 1;
+    pf_off += STEP_BYTES + (wrap ? 7 * (int)strip_bytes : 0);
+    pf_blk = wrap ? 0 : pf_blk + 1;
     HTR_PIN();
   };
 #pragma unroll
@@ -1939,13 +1942,15 @@ __global__ __launch_bounds__(WG_THREADS) void k_anchor_read(const uint32_t* __re
   const uint32_t* wave_base = qw + ((size_t)(rb_first * 8 + w) * nblk + (size_t)c0) * (STEP_BYTES / 4);
   const uint32_t extent = (uint32_t)nsteps * STEP_BYTES + (uint32_t)last_wraps * 7u * strip_bytes;
   const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)wave_base, 0, (int)extent, 0x00020000);
-  int pf_off = lane * 4 * K, pf_blk = c0;
+  const int lane_off = lane * 4 * K;
+  int pf_off = 0, pf_blk = c0;
   StreamRegs<K> buf[P];
   auto prefetch = [&](StreamRegs<K>& dst) {
     HTR_PIN();
-    load_stream_buffer<K>(rsrc, pf_off, dst);
-    pf_off += STEP_BYTES;
-    if (++pf_blk == nblk) { pf_blk = 0; pf_off += 7 * (int)strip_bytes; }
+    load_stream_buffer<K>(rsrc, lane_off + pf_off, dst);
+    const bool wrap = pf_blk == nblk - 1;
+    pf_off += STEP_BYTES + (wrap ? 7 * (int)strip_bytes : 0);
+    pf_blk = wrap ? 0 : pf_blk + 1;
     HTR_PIN();
   };
 #pragma unroll

@@ -327,9 +327,10 @@ def test_captures_can_share_one_workspace(dev):
                 ops.linear(xb, *big)
         torch.cuda.synchronize()
         ops.reserve_capture_workspace(dev, 64 << 20)
-        with torch.cuda.graph(g3):
+        g4 = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g4):
             y3 = ops.linear(xb, *big)
-        g3.replay()
+        g4.replay()
         g1.replay()                              # the earlier graphs still replay against the buffer they recorded
         torch.cuda.synchronize()
         assert torch.equal(y1, want1)

@@ -12,7 +12,8 @@ _CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 LIB_PATH = os.environ.get("HTR_GFX950_LIB") or os.path.join(_CSRC, "libhtr_gfx950.so")
 
 BF16, F16, F32 = 0, 1, 2
-MAX_BATCH = 128
+MAX_BATCH = 2048
+MAX_ROWS_PER_TILE = 128
 MAX_GROUP_ROWS = 32
 MAX_GROUP = 4096
 STATIC_SCRATCH_BYTES = 8 << 20

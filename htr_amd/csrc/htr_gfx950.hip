@@ -285,6 +285,7 @@ struct LinearTail {
   const _Float16* xt_g;   // pre-rotated activations [M][n] f16 (only when PREROT)
   const float* xs_g;      // their sums per (row, block) [M][n/128][4]: even tiles, odd tiles, columns 0..63, columns 64..127
   const float* sc_g;      // per-row activation scale [M]
+  float* tiles;           // GEMM kernel: one 128 x 128 float tile per workgroup for the exchange between column splits
   uint32_t* status;       // workspace word that collects kernel-side failures (bit 0: a finisher gave up waiting)
   unsigned long long chunk_magic;   // ceil(2^40 / chunk): step index -> chunk index
   float cbscale;
@@ -1601,6 +1602,276 @@ __global__ __launch_bounds__(WG_THREADS, MG <= 2 && !ROT ? 4 : 2) void k_linear_
   }
 }
 
+// ------------------------------------------------------------------------------------------------ fused GEMM
+// More than 128 activation rows: the product is bound by the matrix unit, not by the decode, and a wave can no longer hold
+// the accumulators of all rows next to its decode registers.  Here a workgroup owns one 128-row block of the weight, one
+// tile of 128 activation rows and 1/S of the column blocks (grid = S x row blocks x row tiles), and its twelve waves split
+// into two trades that meet once per 128-column block:
+//   producers (waves 0..7)   one 16-row strip each: stream, decode (as in k_linear) and store the block's weights, still
+//                            offset by 1534, as f16 into an LDS tile [128 rows][128 columns]; they also bring the block's
+//                            rotated activations (rotated ahead by a launch of their own) into a second LDS tile
+//                            [128 activation rows][128 columns], requested with the weights, P steps ahead
+//   consumers (waves 8..11)  multiply the tiles of the block before: v_mfma_f32_32x32x16_f16, both operands from LDS, a
+//                            64 x 64 piece of the 128 x 128 output per wave (two operand reads per matrix instruction
+//                            pair: the LDS keeps up with one consumer per SIMD); no memory operations at all
+// Both tiles are double-buffered: while the producers fill tile b the consumers multiply tile b - 1, one barrier per block.
+// The decode runs on the vector unit and the products on the matrix unit of the same SIMDs, so a block costs the longer
+// of the two instead of their sum.  The weight is decoded once per 128 activation rows.
+// Output side as in k_linear_batch: offset removed (1534 x the activation row's sum over the split's columns), activation
+// scale undone, the 128 x 128 output goes to LDS; with S > 1 the last split of a row block collects the others' partials
+// from their slots (they were dispatched earlier) and finishes: row scale, output H128, sign, bias, cast.
+constexpr int GEMM_PRODUCERS = 8, GEMM_CONSUMERS = 4;
+constexpr int GEMM_THREADS = (GEMM_PRODUCERS + GEMM_CONSUMERS) * 64;
+constexpr int GEMM_ROWS = 128;                                 // activation rows per tile
+constexpr int GEMM_LD = 128 + 8;                               // halves per row of an LDS tile: 16-byte rows, 4 banks of shift
+constexpr int GEMM_TILE_HALVES = 128 * GEMM_LD;
+constexpr int GEMM_FIN_LD = 128 + 4;                           // floats per activation row of the output in LDS
+constexpr size_t GEMM_LDS_BYTES = (size_t)4 * GEMM_TILE_HALVES * 2 + 2 * GEMM_ROWS * 4 + 16;     // two W tiles, two X tiles, sums, a flag
+typedef float f16v __attribute__((ext_vector_type(16)));
+
+template <int K, int P>
+__global__ __launch_bounds__(GEMM_THREADS) void k_linear_gemm(const uint32_t* __restrict__ qw, float* __restrict__ part,
+                                                              int m, int n, int M, int S, int flags, const LinearTail t) {
+  extern __shared__ __align__(16) unsigned char lds[];
+  const int lane = threadIdx.x & 63;
+  const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int nblk = n >> 7;
+  const int s_idx = blockIdx.x, rb = blockIdx.y, mt = blockIdx.z;
+  const int j0 = mt * GEMM_ROWS, rows = min(GEMM_ROWS, M - j0);  // this tile's activation rows
+  const int cb = (nblk + S - 1) / S;
+  const int c_begin = s_idx * cb, c_end = min(nblk, c_begin + cb);
+  const int nsteps = c_end - c_begin;                            // >= 1: the host picks S so that no split is empty
+  const int y_dtype = (flags >> 2) & 3;
+  _Float16* w_tile = (_Float16*)lds;                             // [2][128][GEMM_LD]
+  _Float16* x_tile = w_tile + 2 * GEMM_TILE_HALVES;              // [2][128][GEMM_LD]
+  float* s_xs = (float*)(x_tile + 2 * GEMM_TILE_HALVES);         // [2][128]: sum of the block's rotated activations per row
+  float* s_fin = (float*)lds;                                    // [128][GEMM_FIN_LD], over the tiles once the products are done
+  constexpr int OUT_OF_RANGE = 0x7FFFF000;
+  static_assert(P % 2 == 0, "the tile a step goes to must be static in the unrolled loop");
+
+  if (w < GEMM_PRODUCERS) {
+    // ---- producer: strip w of the row block, one step = the 8 tiles under one 128-column block (as in k_linear), and
+    // its share of the block's rotated activations: 16-byte pieces, piece pi = activation row pi / 16, columns
+    // 8 (pi % 16) .. + 7; a thread takes pieces tid, tid + 512, ...; rows beyond M read zeros.  Weights and activations
+    // of a step are requested together, P steps ahead: loads return in order, so a block requested later than the
+    // weights of the steps behind it would hold those up (and the products would wait for a memory round trip per step).
+    constexpr int STEP_BYTES = 256 * K;
+    constexpr int NPT = GEMM_ROWS * 16 / (GEMM_PRODUCERS * 64);      // 4 pieces per thread
+    const int tid = (int)threadIdx.x;
+    const uint32_t* wave_base = qw + ((size_t)(rb * 8 + w) * nblk + (size_t)c_begin) * (STEP_BYTES / 4);
+    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)wave_base, 0, nsteps * STEP_BYTES, 0x00020000);
+    const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)t.xt_g, 0, M * n * 2, 0x00020000);
+    const __amdgpu_buffer_rsrc_t srsrc = __builtin_amdgcn_make_buffer_rsrc((void*)t.xs_g, 0, M * nblk * 16, 0x00020000);
+    int piece_src[NPT], piece_lds[NPT];      // byte offset of the piece in the split's first block, or out of range
+#pragma unroll
+    for (int i = 0; i < NPT; ++i) {
+      const int pi = tid + i * GEMM_PRODUCERS * 64, prow = pi >> 4, pg = pi & 15;
+      piece_src[i] = prow < rows ? ((j0 + prow) * n + c_begin * 128 + pg * 8) * 2 : OUT_OF_RANGE;
+      piece_lds[i] = prow * GEMM_LD + pg * 8;
+    }
+    const int sum_src = tid < rows ? ((j0 + tid) * nblk + c_begin) * 16 : OUT_OF_RANGE;      // {even tiles, odd tiles, ...} of that block
+    const int lane_off = lane * 4 * K;
+    int pf_blk = 0, pf_left = nsteps;        // block (within the split) to request next, steps still to request
+    StreamRegs<K> buf[P];
+    u4 xg[P][NPT];
+    u2 xsg[P];
+    auto prefetch = [&](StreamRegs<K>& dst, u4 (&xd)[NPT], u2& sd) {
+      HTR_PIN();
+      const bool live = pf_left > 0;
+      load_stream_buffer<K>(rsrc, live ? lane_off + pf_blk * STEP_BYTES : OUT_OF_RANGE, dst);
+#pragma unroll
+      for (int i = 0; i < NPT; ++i)
+        xd[i] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, live && piece_src[i] != OUT_OF_RANGE ? piece_src[i] + pf_blk * 256 : OUT_OF_RANGE, 0, 0);
+      sd = __builtin_amdgcn_raw_buffer_load_b64(srsrc, live && sum_src != OUT_OF_RANGE ? sum_src + pf_blk * 16 : OUT_OF_RANGE, 0, 0);
+      ++pf_blk;
+      --pf_left;
+      HTR_PIN();
+    };
+#pragma unroll
+    for (int p = 0; p < P; ++p) prefetch(buf[p], xg[p], xsg[p]);
+    const int hist = history_lane_byteaddr(lane);
+    // lane (tile tl = lane / 8, row pair q = lane % 8) holds rows 2q, 2q + 1 x the tile's 16 columns as four groups of 8
+    _Float16* dst0 = w_tile + (16 * w + 2 * (lane & 7)) * GEMM_LD + 16 * (lane >> 3);
+    auto produce = [&](StreamRegs<K>& sr, u4 (&xd)[NPT], u2& sd, int tile) {
+      DecodedStep<K> d;
+      decode_step<K>(sr, hist, d);
+      _Float16* dst = dst0 + tile * GEMM_TILE_HALVES;
+      *(h8*)dst = d.a[0];
+      *(h8*)(dst + 8) = d.a[1];
+      *(h8*)(dst + GEMM_LD) = d.a[2];
+      *(h8*)(dst + GEMM_LD + 8) = d.a[3];
+#pragma unroll
+      for (int i = 0; i < NPT; ++i) *(u4*)(x_tile + tile * GEMM_TILE_HALVES + piece_lds[i]) = xd[i];
+      if (tid < GEMM_ROWS) s_xs[tile * GEMM_ROWS + tid] = __uint_as_float(sd.x) + __uint_as_float(sd.y);
+      prefetch(sr, xd, sd);
+    };
+    int v = 0;
+    for (; v + P <= nsteps; v += P) {
+#pragma unroll
+      for (int pp = 0; pp < P; ++pp) { produce(buf[pp], xg[pp], xsg[pp], pp & 1); __syncthreads(); }
+    }
+#pragma unroll
+    for (int pp = 0; pp < P; ++pp)
+      if (v + pp < nsteps) { produce(buf[pp], xg[pp], xsg[pp], pp & 1); __syncthreads(); }
+    __syncthreads();                                             // the consumers multiply the last block
+  } else {
+    // ---- consumer c: output rows 64 ih .. + 63 of the row block x activation rows 64 jh .. + 63 of the tile
+    const int c = w - GEMM_PRODUCERS, ih = c >> 1, jh = c & 1;
+    const int l32 = lane & 31, kg = lane >> 5;
+    // activation scale of this lane's two columns of the output (activation rows 64 jh + 32 bb + lane % 32)
+    float scl[2];
+#pragma unroll
+    for (int bb = 0; bb < 2; ++bb) {
+      const int j = 64 * jh + 32 * bb + l32;
+      scl[bb] = j < rows ? ((const HTR_GLOBAL float*)t.sc_g)[j0 + j] : 0.f;
+    }
+    f16v acc[2][2];
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+      for (int bb = 0; bb < 2; ++bb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[a][bb][r] = 0.f;
+    float offs[2] = {0.f, 0.f};                // running 1534 x sum(x~) of this lane's two activation rows
+    // operands of the 32x32x16 instruction: lane (row or column = lane % 32, k-group kg = lane / 32) brings the 8
+    // consecutive k-values 8 kg .. + 7 of its row (weight row) or column (activation row): 16 bytes of an LDS tile row
+    const _Float16* a_lane = w_tile + (64 * ih + l32) * GEMM_LD + 8 * kg;
+    const _Float16* b_lane = x_tile + (64 * jh + l32) * GEMM_LD + 8 * kg;
+    auto multiply = [&](int tile) {
+      const _Float16* ap = a_lane + tile * GEMM_TILE_HALVES;
+      const _Float16* bp = b_lane + tile * GEMM_TILE_HALVES;
+      h8 A[2][2], B[2][2];                     // [k-slice parity][block]: the next slice is read while this one multiplies
+      A[0][0] = *(const h8*)ap; A[0][1] = *(const h8*)(ap + 32 * GEMM_LD);
+      B[0][0] = *(const h8*)bp; B[0][1] = *(const h8*)(bp + 32 * GEMM_LD);
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        const int cur = ks & 1, nxt = cur ^ 1;
+        if (ks + 1 < 8) {
+          A[nxt][0] = *(const h8*)(ap + 16 * (ks + 1)); A[nxt][1] = *(const h8*)(ap + 32 * GEMM_LD + 16 * (ks + 1));
+          B[nxt][0] = *(const h8*)(bp + 16 * (ks + 1)); B[nxt][1] = *(const h8*)(bp + 32 * GEMM_LD + 16 * (ks + 1));
+        }
+#pragma unroll
+        for (int a = 0; a < 2; ++a)
+#pragma unroll
+          for (int bb = 0; bb < 2; ++bb)
+            acc[a][bb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[cur][a], B[cur][bb], acc[a][bb], 0, 0, 0);
+      }
+#pragma unroll
+      for (int bb = 0; bb < 2; ++bb) offs[bb] = __builtin_fmaf(1534.f, s_xs[tile * GEMM_ROWS + 64 * jh + 32 * bb + l32], offs[bb]);
+    };
+    // step it: the producers fill tile it % 2 while the block before it, in the other tile, is multiplied
+    __syncthreads();
+    for (int it = 1; it < nsteps; ++it) {
+      multiply((it - 1) & 1);
+      __syncthreads();
+    }
+    multiply((nsteps - 1) & 1);
+    __syncthreads();                                             // every wave is through with the tiles: the output takes their place
+    // D[i][j]: lane holds column j = lane % 32, register r row i = 8 (r / 4) + 4 (lane / 32) + r % 4 of its 32 x 32 piece
+#pragma unroll
+    for (int a = 0; a < 2; ++a)
+#pragma unroll
+      for (int bb = 0; bb < 2; ++bb) {
+        float* dst = s_fin + (64 * jh + 32 * bb + l32) * GEMM_FIN_LD + 64 * ih + 32 * a + 4 * kg;
+#pragma unroll
+        for (int rq = 0; rq < 4; ++rq)
+          *(f4*)(dst + 8 * rq) = f4{(acc[a][bb][4 * rq] - offs[bb]) * scl[bb], (acc[a][bb][4 * rq + 1] - offs[bb]) * scl[bb],
+                                    (acc[a][bb][4 * rq + 2] - offs[bb]) * scl[bb], (acc[a][bb][4 * rq + 3] - offs[bb]) * scl[bb]};
+      }
+  }
+  __syncthreads();
+
+  // ---- exchange between the splits of a row block.  A split's 128 x 128 partial is too large to hand over word by word
+  // with in-band markers (the finisher would pay a memory round trip per row): the partial goes to the workgroup's tile
+  // in the scratch half of the workspace with device-scope stores, and ONE flag word per workgroup, set after every
+  // thread's stores have completed, says it is there.  The last split (dispatched after the others, so waiting for
+  // them cannot deadlock; bounded all the same) waits for the flags, adds the tiles to its own in LDS and clears the flags.
+  constexpr int WAVES = GEMM_PRODUCERS + GEMM_CONSUMERS;
+  const size_t wg0 = ((size_t)mt * gridDim.y + rb) * S;              // index of split 0's workgroup of this (row block, tile)
+  uint32_t* ready = (uint32_t*)part;                                 // one word per workgroup, zero between launches
+  float* tiles = t.tiles;                                            // [workgroups][128][128] floats in the scratch half of the workspace
+  uint32_t& s_failed = *(uint32_t*)(s_xs + 2 * GEMM_ROWS);       // the finisher's wait gave up (behind the sums: not overlaid by the output)
+  if (S > 1) {
+    typedef unsigned long long u64;
+    if (s_idx != S - 1) {
+      u64* dst = (u64*)(tiles + (wg0 + s_idx) * (size_t)(GEMM_ROWS * 128));
+      for (int idx = threadIdx.x; idx < rows * 64; idx += GEMM_THREADS) {
+        const f2 v = *(const f2*)(s_fin + (idx >> 6) * GEMM_FIN_LD + 2 * (idx & 63));
+        __hip_atomic_store(dst + idx, __builtin_bit_cast(u64, v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");             // this thread's stores have completed, device-wide
+      __syncthreads();
+      if (threadIdx.x == 0) __hip_atomic_store(ready + wg0 + s_idx, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      return;
+    }
+    if (w == 0) {
+      bool failed = false;
+      int tries = 0;
+      for (;;) {
+        const uint32_t f = lane < S - 1 ? __hip_atomic_load(ready + wg0 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 1u;
+        if (!__any(f == 0u)) break;
+        if (++tries >= t.spin_limit) { failed = true; break; }
+        __builtin_amdgcn_s_sleep(8);
+      }
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+      if (lane == 0) {
+        s_failed = failed ? 1u : 0u;
+        if (failed) report_give_up(t.status);
+      }
+    }
+    __syncthreads();
+    if (s_failed == 0u) {
+      // own tile += the other splits' tiles: a thread's pieces (8 bytes each) of every contributor are requested together,
+      // so the sum costs a few memory round trips, not one per contributor
+      const u64* src = (const u64*)(tiles + wg0 * (size_t)(GEMM_ROWS * 128));
+      for (int base = threadIdx.x; base < rows * 64; base += 4 * GEMM_THREADS) {
+        u64 got[7][4];
+#pragma unroll
+        for (int k = 0; k < 7; ++k)
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const int idx = base + u * GEMM_THREADS;
+            got[k][u] = k < S - 1 && idx < rows * 64
+                            ? __hip_atomic_load(src + (size_t)k * (GEMM_ROWS * 64) + idx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0ull;
+          }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int idx = base + u * GEMM_THREADS;
+          if (idx < rows * 64) {
+            f2* own = (f2*)(s_fin + (idx >> 6) * GEMM_FIN_LD + 2 * (idx & 63));
+            f2 sum = *own;
+#pragma unroll
+            for (int k = 0; k < 7; ++k) { const f2 g = __builtin_bit_cast(f2, got[k][u]); sum.x += g.x; sum.y += g.y; }
+            *own = sum;
+          }
+        }
+      }
+      if (threadIdx.x < S - 1) __hip_atomic_store(ready + wg0 + threadIdx.x, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+  }
+
+  // ---- output side, one activation row per wave and turn; lane holds output rows lane and lane + 64 of the row block
+  const bool failed = load_status(t.status) != 0u || (S > 1 && s_failed != 0u);   // also: an earlier launch on this workspace gave up
+  const int r0 = rb * 128 + lane, r1 = r0 + 64;
+  const float rs0 = f16_bits_to_float(((const HTR_GLOBAL uint16_t*)t.scales)[r0]) * t.cbscale * INV_SQRT128;
+  const float rs1 = f16_bits_to_float(((const HTR_GLOBAL uint16_t*)t.scales)[r1]) * t.cbscale * INV_SQRT128;
+  const float sg0 = ((((const HTR_GLOBAL uint8_t*)t.sv)[r0 >> 3] >> (lane & 7)) & 1u) ? -1.f : 1.f;
+  const float sg1 = ((((const HTR_GLOBAL uint8_t*)t.sv)[r1 >> 3] >> (lane & 7)) & 1u) ? -1.f : 1.f;
+  float b0v = 0.f, b1v = 0.f;
+  if (t.bias != nullptr) { b0v = load_elem_g(t.bias, y_dtype, r0); b1v = load_elem_g(t.bias, y_dtype, r1); }
+  for (int j = w; j < rows; j += WAVES) {
+    const float* own = s_fin + j * GEMM_FIN_LD;
+    float v0s = own[lane] * rs0, v1s = own[lane + 64] * rs1;
+    fwht128_wave(v0s, v1s, lane);
+    v0s = __builtin_fmaf(v0s, sg0, b0v);
+    v1s = __builtin_fmaf(v1s, sg1, b1v);
+    if (failed) { v0s = __builtin_nanf(""); v1s = v0s; }
+    store_elem_g(t.y, y_dtype, (size_t)(j0 + j) * m + r0, v0s);
+    store_elem_g(t.y, y_dtype, (size_t)(j0 + j) * m + r1, v1s);
+  }
+}
+
 // ------------------------------------------------------------------------------------------------ debug decodes
 template <int K, int U> struct ForEach32 {
   template <typename F> __device__ __forceinline__ static void run(const Window<K>& w, F&& f) {
@@ -2288,6 +2559,36 @@ inline bool make_batch_plan(int m, int n, int M, int want_S, BatchPlan& bp) {
   return found;
 }
 
+// ---- GEMM kernel (more than 128 rows): tiles of 128 activation rows in the grid's z, split S of the column blocks while the
+// grid stays within one workgroup per compute unit (its 137 KB of LDS leave room for one)
+struct GemmPlan { int S, cb, mtiles, wgs; };
+constexpr int GEMM_MIN_M = HTR_MAX_ROWS_PER_TILE + 1;       // rows from which the library policy takes the GEMM kernel
+inline bool make_gemm_plan(int m, int n, int M, int want_S, GemmPlan& gp) {
+  const int nblk = n / 128, rbs = m / 128;
+  if ((long)M * n * 2 >= (1L << 31)) return false;          // the kernel addresses the rotated activations with 32-bit byte offsets
+  gp.mtiles = (M + GEMM_ROWS - 1) / GEMM_ROWS;
+  if (gp.mtiles > 65535) return false;
+  const long base = (long)rbs * gp.mtiles;
+  const int cus = num_cu();
+  const int by_cus = cus / base > 1 ? (int)(cus / base) : 1;
+  const int limit = want_S > 0 ? want_S : (by_cus < 8 ? by_cus : 8);
+  bool found = false;
+  for (int S = 1; S <= nblk && S <= limit && S <= 8; ++S) {
+    const int cb = (nblk + S - 1) / S;
+    if ((nblk + cb - 1) / cb != S) continue;                       // some split would be empty
+    if (want_S > 0 && S != want_S) continue;
+    gp.S = S; gp.cb = cb; gp.wgs = (int)(base * S); found = true;
+  }
+  return found;
+}
+// workspace of the GEMM kernel: one flag word per workgroup in the zeroed half; rotated activations and the exchange tiles
+// (only with column splits) in the scratch half
+inline size_t gemm_scratch_bytes(int n, int M, const GemmPlan& gp) {
+  return prerot_bytes(n, M) + (gp.S > 1 ? (size_t)gp.wgs * GEMM_ROWS * 128 * sizeof(float) : 0);
+}
+// nsplit bit 28: the GEMM kernel with the split in the low bits (0 = its own policy); otherwise from GEMM_MIN_M rows
+inline bool wants_gemm(int M, int nsplit) { return nsplit > 0 ? (nsplit & (1 << 28)) != 0 : M >= GEMM_MIN_M; }
+
 struct BatchArgs { const uint32_t* qw; float* part; const void* x; const uint8_t* su; int m, n, M, flags; };
 template <int K, int MB, bool ROT> int launch_batch_v(const BatchArgs& a, const LinearTail& t, const BatchPlan& bp, hipStream_t st) {
   const size_t lds = balanced_lds_request(bp.lds, bp.wgs);
@@ -2311,6 +2612,7 @@ template <int K> int launch_batch_k(const BatchArgs& a, bool rot, const LinearTa
 // A matrix whose splits are four column blocks or fewer on a full grid (4096x4096: 8 splits of 4 blocks) is also ahead
 // with the batched kernel at 7 and 8 rows, when its workgroups rotate their own slices (8 rows: 9.2 against 10.4 us).
 inline bool wants_batch(int M, int nsplit, int m, int n) {
+  if (wants_gemm(M, nsplit)) return false;
   if (nsplit > 0) return (nsplit & (1 << 29)) != 0;
   if (M >= BATCH_MIN_M || (M >= 6 && m / 128 >= 192)) return true;
   if (M >= 7) {
@@ -2356,7 +2658,7 @@ const char* htr_strerror(int status) {
     case HTR_ERR_NULL: return "a required pointer is NULL";
     case HTR_ERR_K: return "unsupported K (HTR-W1 allows 2..8)";
     case HTR_ERR_SHAPE: return "m and n must be positive multiples of 128";
-    case HTR_ERR_BATCH: return "M must be in 1..128 for one launch (1..32 for a grouped problem or an explicit chunked plan)";
+    case HTR_ERR_BATCH: return "M must be in 1..2048 for one launch (1..128 for an explicit chunked or batched plan, 1..32 for a grouped problem)";
     case HTR_ERR_DTYPE: return "dtype must be bf16 (0), f16 (1) or f32 (2)";
     case HTR_ERR_WORKSPACE: return "workspace too small or not 256-byte aligned";
     case HTR_ERR_ALIGN: return "tensor pointer not aligned (qweight 16 B, others natural)";
@@ -2373,6 +2675,12 @@ float htr_cbscale(void) { return (float)(1.0 / __builtin_sqrt(MEAN_SQ)); }
 
 size_t htr_workspace_bytes(int m, int n, int K, int M, int nsplit) {
   if (K < 2 || K > 8 || !shape_ok(m, n) || M < 1 || M > HTR_MAX_BATCH) return 0;
+  if (wants_gemm(M, nsplit)) {
+    GemmPlan gp;
+    if (!make_gemm_plan(m, n, M, nsplit > 0 ? nsplit & 0xFFFFF : 0, gp)) return 0;
+    return ws_need((size_t)gp.wgs * sizeof(uint32_t), gemm_scratch_bytes(n, M, gp));
+  }
+  if (M > HTR_MAX_ROWS_PER_TILE) return 0;       // the other kernels take up to 128 rows
   if (wants_batch(M, nsplit, m, n)) {
     BatchPlan bp;
     if (!make_batch_plan(m, n, M, nsplit > 0 ? nsplit & 0xFFFFF : 0, bp)) return 0;
@@ -2389,6 +2697,13 @@ int htr_linear_plan(int m, int n, int K, int M, int nsplit, int* out6) {
   if (K < 2 || K > 8) return HTR_ERR_K;
   if (!shape_ok(m, n)) return HTR_ERR_SHAPE;
   if (M < 1 || M > HTR_MAX_BATCH) return HTR_ERR_BATCH;
+  if (wants_gemm(M, nsplit)) {
+    GemmPlan gp;
+    if (!make_gemm_plan(m, n, M, nsplit > 0 ? nsplit & 0xFFFFF : 0, gp)) return HTR_ERR_SPLIT;
+    out6[0] = gp.cb; out6[1] = gp.wgs; out6[2] = gp.mtiles; out6[3] = gp.S; out6[4] = 1; out6[5] = (int)GEMM_LDS_BYTES;
+    return HTR_OK;
+  }
+  if (M > HTR_MAX_ROWS_PER_TILE) return HTR_ERR_BATCH;
   if (wants_batch(M, nsplit, m, n)) {
     BatchPlan bp;
     if (!make_batch_plan(m, n, M, nsplit > 0 ? nsplit & 0xFFFFF : 0, bp)) return HTR_ERR_SPLIT;
@@ -2441,6 +2756,47 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
   if (((uintptr_t)qweight & 15) || ((uintptr_t)scales & 1) || ((uintptr_t)x & (x_dtype == HTR_F32 ? 3 : 1)) ||
       ((uintptr_t)y & (y_dtype == HTR_F32 ? 3 : 1)) || (bias && ((uintptr_t)bias & (y_dtype == HTR_F32 ? 3 : 1))))
     return HTR_ERR_ALIGN;
+  if (wants_gemm(M, nsplit)) {
+    GemmPlan gp;
+    if (!make_gemm_plan(m, n, M, nsplit > 0 ? nsplit & 0xFFFFF : 0, gp)) return HTR_ERR_SPLIT;
+    const size_t need = htr_workspace_bytes(m, n, K, M, nsplit);
+    if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255)) return HTR_ERR_WORKSPACE;
+    unsigned char* wsp = (unsigned char*)workspace + ws_half(workspace_bytes);
+    LinearTail t;
+    t.scales = (const uint16_t*)scales; t.sv = (const uint8_t*)sv; t.bias = bias; t.y = y;
+    t.xt_g = (const _Float16*)wsp;
+    t.xs_g = (const float*)(wsp + align256((size_t)M * n * 2));
+    t.sc_g = (const float*)(wsp + align256((size_t)M * n * 2) + align256((size_t)M * (n / 128) * 16));
+    t.tiles = (float*)(wsp + prerot_bytes(n, M));
+    t.status = (uint32_t*)workspace;
+    t.cbscale = htr_cbscale();
+    t.spin_limit = g_spin_limit.load(std::memory_order_relaxed);
+    t.chunk_magic = 0;
+    t.group = nullptr; t.group_prerot_stride = 0; t.group_part_stride = 0;
+    hipStream_t st = (hipStream_t)stream;
+    HTR_CHECK_HIP(launch_rotation(x, (const uint8_t*)su, n, M, x_dtype, t, st));
+    const uint32_t* qwp = (const uint32_t*)qweight;
+    float* flags = (float*)((unsigned char*)workspace + WS_HEADER);
+    const int flg = x_dtype | (y_dtype << 2);
+#define HTR_LAUNCH_GEMM(KK_, PP_)                                                                                          \
+    {                                                                                                                      \
+      HTR_CHECK_HIP((allow_full_lds<k_linear_gemm<KK_, PP_>>()));                                                          \
+      HTR_CHECK_HIP(launch_kernel(k_linear_gemm<KK_, PP_>, dim3(gp.S, m / 128, gp.mtiles), dim3(GEMM_THREADS), GEMM_LDS_BYTES, st, \
+                                  qwp, flags, m, n, M, gp.S, flg, t));                                                     \
+    }
+    switch (K) {
+      case 2: HTR_LAUNCH_GEMM(2, 4); break;
+      case 3: HTR_LAUNCH_GEMM(3, 4); break;
+      case 4: HTR_LAUNCH_GEMM(4, 4); break;
+      case 5: HTR_LAUNCH_GEMM(5, 2); break;
+      case 6: HTR_LAUNCH_GEMM(6, 2); break;
+      case 7: HTR_LAUNCH_GEMM(7, 2); break;
+      default: HTR_LAUNCH_GEMM(8, 2); break;
+    }
+#undef HTR_LAUNCH_GEMM
+    return HTR_OK;
+  }
+  if (M > HTR_MAX_ROWS_PER_TILE) return HTR_ERR_BATCH;        // explicit plans of the other kernels take up to 128 rows
   if (wants_batch(M, nsplit, m, n)) {
     BatchPlan bp;
     if (!make_batch_plan(m, n, M, nsplit > 0 ? nsplit & 0xFFFFF : 0, bp)) return HTR_ERR_SPLIT;
@@ -2456,7 +2812,7 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
     t.cbscale = htr_cbscale();
     t.spin_limit = g_spin_limit.load(std::memory_order_relaxed);
     t.chunk_magic = 0;
-    t.group = nullptr; t.group_prerot_stride = 0; t.group_part_stride = 0;
+    t.group = nullptr; t.group_prerot_stride = 0; t.group_part_stride = 0; t.tiles = nullptr;
     hipStream_t st = (hipStream_t)stream;
     // the workgroups rotate their own activations where the plan allows it (16-bit rows on 16-byte boundaries)
     const bool rot = bp.rot && x_dtype != HTR_F32 && ((uintptr_t)x & 15) == 0;
@@ -2498,7 +2854,7 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
   t.status = (uint32_t*)workspace;
   t.cbscale = htr_cbscale();
   t.spin_limit = g_spin_limit.load(std::memory_order_relaxed);
-  t.group = nullptr; t.group_prerot_stride = 0; t.group_part_stride = 0;
+  t.group = nullptr; t.group_prerot_stride = 0; t.group_part_stride = 0; t.tiles = nullptr;
   t.chunk_magic = (((unsigned long long)1 << 40) + (unsigned)pl.chunk - 1) / (unsigned)pl.chunk;
   hipStream_t st = (hipStream_t)stream;
   if (prerot) {
@@ -2607,6 +2963,7 @@ int htr_linear_grouped(const htr_group_entry* entries, int count, int m, int n, 
   t.cbscale = htr_cbscale();
   t.spin_limit = g_spin_limit.load(std::memory_order_relaxed);
   t.chunk_magic = (((unsigned long long)1 << 40) + (unsigned)pl.chunk - 1) / (unsigned)pl.chunk;
+  t.tiles = nullptr;
   t.group = entries; t.group_prerot_stride = pre; t.group_part_stride = (unsigned long long)pl.wgs * max_M * 128;
   hipStream_t st = (hipStream_t)stream;
   HTR_CHECK_HIP(launch_kernel(k_rotate, dim3((n / 128 + WG_WAVES - 1) / WG_WAVES, max_M, count), dim3(WG_THREADS), 0, st, (const void*)nullptr,
@@ -2642,7 +2999,7 @@ int htr_anchor_linear(int kind, const void* qweight, const void* scales, const v
   t.status = (uint32_t*)workspace;
   t.cbscale = htr_cbscale();
   t.spin_limit = g_spin_limit.load(std::memory_order_relaxed);
-  t.group = nullptr; t.group_prerot_stride = 0; t.group_part_stride = 0;
+  t.group = nullptr; t.group_prerot_stride = 0; t.group_part_stride = 0; t.tiles = nullptr;
   t.chunk_magic = (((unsigned long long)1 << 40) + (unsigned)pl.chunk - 1) / (unsigned)pl.chunk;
   hipStream_t st = (hipStream_t)stream;
   const size_t lds = balanced_lds_request(pl.lds, pl.wgs);

@@ -43,7 +43,8 @@ typedef enum {
 /* element type codes; same numbering as the reference's out-dtype map (htr/ops.py:79,94) */
 enum { HTR_BF16 = 0, HTR_F16 = 1, HTR_F32 = 2 };
 
-#define HTR_MAX_BATCH 128       /* activation rows one htr_linear launch accepts */
+#define HTR_MAX_BATCH 2048      /* activation rows one htr_linear launch accepts */
+#define HTR_MAX_ROWS_PER_TILE 128   /* up to here one workgroup holds all rows; beyond, the GEMM kernel works in tiles of 128 rows */
 #define HTR_MAX_GROUP_ROWS 32   /* rows per problem of htr_linear_grouped (and of an explicit chunked plan, see nsplit) */
 #define HTR_MAX_GROUP 4096 /* problems one htr_linear_grouped launch accepts */
 

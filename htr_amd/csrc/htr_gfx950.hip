@@ -1603,38 +1603,42 @@ __global__ __launch_bounds__(WG_THREADS, MG <= 2 && !ROT ? 4 : 2) void k_linear_
 }
 
 // ------------------------------------------------------------------------------------------------ fused GEMM
-// More than 128 activation rows: the product is bound by the matrix unit, not by the decode, and a wave can no longer hold
-// the accumulators of all rows next to its decode registers.  Here a workgroup owns one 128-row block of the weight, one
-// tile of 128 activation rows and 1/S of the column blocks (grid = S x row blocks x row tiles), and its twelve waves split
-// into two trades that meet once per 128-column block:
-//   producers (waves 0..7)   one 16-row strip each: stream, decode (as in k_linear) and store the block's weights, still
-//                            offset by 1534, as f16 into an LDS tile [128 rows][128 columns]; they also bring the block's
-//                            rotated activations (rotated ahead by a launch of their own) into a second LDS tile
-//                            [128 activation rows][128 columns], requested with the weights, P steps ahead
-//   consumers (waves 8..11)  multiply the tiles of the block before: v_mfma_f32_32x32x16_f16, both operands from LDS, a
-//                            64 x 64 piece of the 128 x 128 output per wave (two operand reads per matrix instruction
-//                            pair: the LDS keeps up with one consumer per SIMD); no memory operations at all
-// Both tiles are double-buffered: while the producers fill tile b the consumers multiply tile b - 1, one barrier per block.
-// The decode runs on the vector unit and the products on the matrix unit of the same SIMDs, so a block costs the longer
-// of the two instead of their sum.  The weight is decoded once per 128 activation rows.
-// Output side as in k_linear_batch: offset removed (1534 x the activation row's sum over the split's columns), activation
-// scale undone, the 128 x 128 output goes to LDS; with S > 1 the last split of a row block collects the others' partials
-// from their slots (they were dispatched earlier) and finishes: row scale, output H128, sign, bias, cast.
-constexpr int GEMM_PRODUCERS = 8, GEMM_CONSUMERS = 4;
-constexpr int GEMM_THREADS = (GEMM_PRODUCERS + GEMM_CONSUMERS) * 64;
-constexpr int GEMM_ROWS = 128;                                 // activation rows per tile
-constexpr int GEMM_LD = 128 + 8;                               // halves per row of an LDS tile: 16-byte rows, 4 banks of shift
-constexpr int GEMM_TILE_HALVES = 128 * GEMM_LD;
+// More than 128 activation rows: the product is bound by the matrix unit and by what feeds it, not by the decode.  A
+// workgroup owns one 128-row block of the weight, one tile of 128 activation rows and 1/S of the column blocks (grid =
+// S x row blocks x row tiles).  Per 128-column block, wave w = (row half rh = w % 2, column quarter cq = w / 2) decodes 64
+// rows x 32 columns: its lanes take the (tile, row pair) granules of strips 4 rh .. 4 rh + 3 in tile columns 2 cq (lanes
+// 0..31) and 2 cq + 1 (lanes 32..63).  A granule is rows 2q, 2q + 1 x the tile's 16 columns; the 32x32x16 matrix
+// instruction wants lane (row i = lane % 32, k-group lane / 32) to bring 8 consecutive columns of ONE row, the two
+// k-groups of a row in lanes l and l + 32.  One v_permlane32_swap per register moves "columns 8..15 of the lower lanes'
+// granule" up and "columns 0..7 of the upper lanes' granule" down, after which the decode registers ARE the A operands:
+// (even rows | odd rows) x (tile column 2 cq | 2 cq + 1), 32 weight rows each.  The weights never pass through LDS.
+// The B operands are the block's rotated activations (rotated ahead by a launch of their own), staged through LDS in
+// three buffers; each B read (32 activation rows x 16 columns) serves two matrix instructions (even and odd rows), 0.5 KB
+// of LDS traffic per instruction: half of what a design with both operands in LDS needs, which is what the LDS can
+// sustain next to the staging.  The decode of the next block is interleaved with the matrix instructions of this one.
+// Output side: every wave has the partial of its 64 rows over its 32 columns; the four column quarters meet in LDS, the
+// offset (1534 x the activation row's sum over the split's columns) is removed by the first quarter, the activation scale
+// is undone; with S > 1 the last split of a row block collects the others' tiles and finishes: row scale, output H128,
+// sign, bias, cast.
+constexpr int GEMM_THREADS = WG_THREADS;
+constexpr int GEMM_JB = 3;                                     // 32-row blocks of activation rows per tile
+constexpr int GEMM_ROWS = 32 * GEMM_JB;                        // activation rows per tile
+constexpr int GEMM_LD = 128 + 8;                               // halves per row of a staged activation block: 16-byte rows, 4 banks of shift
+constexpr int GEMM_TILE_HALVES = GEMM_ROWS * GEMM_LD;
+constexpr int GEMM_XBUFS = 3;
 constexpr int GEMM_FIN_LD = 128 + 4;                           // floats per activation row of the output in LDS
-constexpr size_t GEMM_LDS_BYTES = (size_t)4 * GEMM_TILE_HALVES * 2 + 2 * GEMM_ROWS * 4 + 16;     // two W tiles, two X tiles, sums, a flag
+constexpr size_t GEMM_FIN_BYTES = (size_t)2 * GEMM_ROWS * GEMM_FIN_LD * 4;            // two copies of the output (column quarters 0, 2 | 1, 3)
+constexpr size_t GEMM_X_BYTES = (size_t)GEMM_XBUFS * GEMM_TILE_HALVES * 2 + GEMM_XBUFS * GEMM_ROWS * 4;
+constexpr size_t GEMM_LDS_BYTES = (GEMM_FIN_BYTES > GEMM_X_BYTES ? GEMM_FIN_BYTES : GEMM_X_BYTES) + 16;
 typedef float f16v __attribute__((ext_vector_type(16)));
 
 template <int K, int P>
 __global__ __launch_bounds__(GEMM_THREADS) void k_linear_gemm(const uint32_t* __restrict__ qw, float* __restrict__ part,
-                                                              int m, int n, int M, int S, int flags, const LinearTail t) {
+                                                                 int m, int n, int M, int S, int flags, const LinearTail t) {
   extern __shared__ __align__(16) unsigned char lds[];
   const int lane = threadIdx.x & 63;
   const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int rh = w & 1, cq = w >> 1;
   const int nblk = n >> 7;
   const int s_idx = blockIdx.x, rb = blockIdx.y, mt = blockIdx.z;
   const int j0 = mt * GEMM_ROWS, rows = min(GEMM_ROWS, M - j0);  // this tile's activation rows
@@ -1642,142 +1646,202 @@ __global__ __launch_bounds__(GEMM_THREADS) void k_linear_gemm(const uint32_t* __
   const int c_begin = s_idx * cb, c_end = min(nblk, c_begin + cb);
   const int nsteps = c_end - c_begin;                            // >= 1: the host picks S so that no split is empty
   const int y_dtype = (flags >> 2) & 3;
-  _Float16* w_tile = (_Float16*)lds;                             // [2][128][GEMM_LD]
-  _Float16* x_tile = w_tile + 2 * GEMM_TILE_HALVES;              // [2][128][GEMM_LD]
-  float* s_xs = (float*)(x_tile + 2 * GEMM_TILE_HALVES);         // [2][128]: sum of the block's rotated activations per row
-  float* s_fin = (float*)lds;                                    // [128][GEMM_FIN_LD], over the tiles once the products are done
+  _Float16* x_tile = (_Float16*)lds;                             // [3][128][GEMM_LD]
+  float* s_xs = (float*)(x_tile + GEMM_XBUFS * GEMM_TILE_HALVES);   // [3][128]: sum of the block's rotated activations per row
+  float* s_fin = (float*)lds;                                    // [2][128][GEMM_FIN_LD], over the blocks once the products are done
+  uint32_t& s_failed = *(uint32_t*)(lds + GEMM_LDS_BYTES - 16);  // the finisher's wait gave up
   constexpr int OUT_OF_RANGE = 0x7FFFF000;
-  static_assert(P % 2 == 0, "the tile a step goes to must be static in the unrolled loop");
+  const int l32 = lane & 31, kg = lane >> 5;
 
-  if (w < GEMM_PRODUCERS) {
-    // ---- producer: strip w of the row block, one step = the 8 tiles under one 128-column block (as in k_linear), and
-    // its share of the block's rotated activations: 16-byte pieces, piece pi = activation row pi / 16, columns
-    // 8 (pi % 16) .. + 7; a thread takes pieces tid, tid + 512, ...; rows beyond M read zeros.  Weights and activations
-    // of a step are requested together, P steps ahead: loads return in order, so a block requested later than the
-    // weights of the steps behind it would hold those up (and the products would wait for a memory round trip per step).
-    constexpr int STEP_BYTES = 256 * K;
-    constexpr int NPT = GEMM_ROWS * 16 / (GEMM_PRODUCERS * 64);      // 4 pieces per thread
-    const int tid = (int)threadIdx.x;
-    const uint32_t* wave_base = qw + ((size_t)(rb * 8 + w) * nblk + (size_t)c_begin) * (STEP_BYTES / 4);
-    const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)wave_base, 0, nsteps * STEP_BYTES, 0x00020000);
-    const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)t.xt_g, 0, M * n * 2, 0x00020000);
-    const __amdgpu_buffer_rsrc_t srsrc = __builtin_amdgcn_make_buffer_rsrc((void*)t.xs_g, 0, M * nblk * 16, 0x00020000);
-    int piece_src[NPT], piece_lds[NPT];      // byte offset of the piece in the split's first block, or out of range
+  // ---- staging of the rotated activations: 16-byte pieces, piece pi = activation row pi / 16, columns 8 (pi % 16) .. + 7;
+  // a thread takes pieces tid, tid + 512, ...; rows beyond M read zeros.  A block is requested three steps before its use, in
+  // two register sets: loads return in order, so behind the weight requests of the steps ahead (which take a trip to
+  // memory) a block needs as long as they do, however close it sits in the L2.
+  constexpr int NPT = GEMM_ROWS * 16 / GEMM_THREADS;               // pieces per thread
+  const int tid = (int)threadIdx.x;
+  const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)t.xt_g, 0, M * n * 2, 0x00020000);
+  const __amdgpu_buffer_rsrc_t srsrc = __builtin_amdgcn_make_buffer_rsrc((void*)t.xs_g, 0, M * nblk * 16, 0x00020000);
+  int piece_src[NPT], piece_lds[NPT];
 #pragma unroll
-    for (int i = 0; i < NPT; ++i) {
-      const int pi = tid + i * GEMM_PRODUCERS * 64, prow = pi >> 4, pg = pi & 15;
-      piece_src[i] = prow < rows ? ((j0 + prow) * n + c_begin * 128 + pg * 8) * 2 : OUT_OF_RANGE;
-      piece_lds[i] = prow * GEMM_LD + pg * 8;
+  for (int i = 0; i < NPT; ++i) {
+    const int pi = tid + i * GEMM_THREADS, prow = pi >> 4, pg = pi & 15;
+    piece_src[i] = prow < rows ? ((j0 + prow) * n + pg * 8) * 2 : -1;
+    piece_lds[i] = prow * GEMM_LD + pg * 8;
+  }
+  const int sum_src = tid < rows ? ((j0 + tid) * nblk) * 16 : -1;          // {even tiles, odd tiles, ...} of block 0
+  u4 xg[2][NPT];
+  u2 xsg[2];
+  auto stage_load = [&](int blk, int set) {    // block index in the row; beyond the split: zeros, no traffic
+    HTR_PIN();
+    const bool live = blk < c_end;
+#pragma unroll
+    for (int i = 0; i < NPT; ++i)
+      xg[set][i] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, live && piece_src[i] >= 0 ? piece_src[i] + blk * 256 : OUT_OF_RANGE, 0, 0);
+    xsg[set] = __builtin_amdgcn_raw_buffer_load_b64(srsrc, live && sum_src >= 0 ? sum_src + blk * 16 : OUT_OF_RANGE, 0, 0);
+    HTR_PIN();
+  };
+  auto stage_store = [&](int xb, int set) {
+#pragma unroll
+    for (int i = 0; i < NPT; ++i) *(u4*)(x_tile + xb * GEMM_TILE_HALVES + piece_lds[i]) = xg[set][i];
+    if (tid < GEMM_ROWS) s_xs[xb * GEMM_ROWS + tid] = __uint_as_float(xsg[set].x) + __uint_as_float(xsg[set].y);
+  };
+  stage_load(c_begin, 0);
+  stage_load(c_begin + 1, 1);
+
+  // ---- the weight stream: lane = (tile column 2 cq + lane / 32, strip 4 rh + lane % 32 / 8, row pair q = lane % 8); the 8
+  // lanes of a tile are consecutive, so the history exchange is the one of k_linear.  One descriptor over the row block's
+  // eight strips from the split's first byte on; a request beyond the split's last block is sent out of range.
+  constexpr int STEP_BYTES = 256 * K;
+  const uint32_t strip_bytes = (uint32_t)nblk * STEP_BYTES;
+  const uint32_t* base = qw + ((size_t)(rb * 8) * nblk + (size_t)c_begin) * (STEP_BYTES / 4);
+  const __amdgpu_buffer_rsrc_t rsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, (int)(7u * strip_bytes + (uint32_t)nsteps * STEP_BYTES), 0x00020000);
+  const int lane_off = (4 * rh + (l32 >> 3)) * (int)strip_bytes + ((2 * cq + kg) * 8 + (lane & 7)) * 4 * K;
+  int pf_off = 0, pf_left = nsteps;
+  StreamRegs<K> buf[P];
+  auto prefetch = [&](StreamRegs<K>& dst) {
+    HTR_PIN();
+    load_stream_buffer<K>(rsrc, pf_left > 0 ? lane_off + pf_off : OUT_OF_RANGE, dst);
+    pf_off += STEP_BYTES;
+    --pf_left;
+    HTR_PIN();
+  };
+#pragma unroll
+  for (int p = 0; p < P; ++p) prefetch(buf[p]);
+  const int hist = history_lane_byteaddr(lane);
+
+  // A operands of one step, after the swap: [even | odd rows][tile column 2 cq | 2 cq + 1]
+  struct Operands { h8 a[2][2]; };
+  auto form = [&](const DecodedStep<K>& d, Operands& o) {
+    // d.a[0], d.a[1] = row 2q columns 0..7, 8..15; d.a[2], d.a[3] = row 2q + 1 columns 0..7, 8..15 of the lane's tile
+#pragma unroll
+    for (int par = 0; par < 2; ++par) {
+      const u4 lo = __builtin_bit_cast(u4, d.a[2 * par]), hi = __builtin_bit_cast(u4, d.a[2 * par + 1]);
+      u4 t0, t1;
+#pragma unroll
+      for (int dw = 0; dw < 4; ++dw) {
+        // x: lo with its upper lanes replaced by hi's lower lanes; y: hi with its lower lanes replaced by lo's upper lanes
+        const u2s r = __builtin_amdgcn_permlane32_swap(lo[dw], hi[dw], false, false);
+        t0[dw] = r.x; t1[dw] = r.y;
+      }
+      o.a[par][0] = __builtin_bit_cast(h8, t0);
+      o.a[par][1] = __builtin_bit_cast(h8, t1);
     }
-    const int sum_src = tid < rows ? ((j0 + tid) * nblk + c_begin) * 16 : OUT_OF_RANGE;      // {even tiles, odd tiles, ...} of that block
-    const int lane_off = lane * 4 * K;
-    int pf_blk = 0, pf_left = nsteps;        // block (within the split) to request next, steps still to request
-    StreamRegs<K> buf[P];
-    u4 xg[P][NPT];
-    u2 xsg[P];
-    auto prefetch = [&](StreamRegs<K>& dst, u4 (&xd)[NPT], u2& sd) {
-      HTR_PIN();
-      const bool live = pf_left > 0;
-      load_stream_buffer<K>(rsrc, live ? lane_off + pf_blk * STEP_BYTES : OUT_OF_RANGE, dst);
+  };
+
+  // activation scale of this lane's column of each 32-row block of the output (activation row 32 jb + lane % 32)
+  constexpr int JB = GEMM_ROWS / 32;
+  f16v acc[JB][2];
 #pragma unroll
-      for (int i = 0; i < NPT; ++i)
-        xd[i] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, live && piece_src[i] != OUT_OF_RANGE ? piece_src[i] + pf_blk * 256 : OUT_OF_RANGE, 0, 0);
-      sd = __builtin_amdgcn_raw_buffer_load_b64(srsrc, live && sum_src != OUT_OF_RANGE ? sum_src + pf_blk * 16 : OUT_OF_RANGE, 0, 0);
-      ++pf_blk;
-      --pf_left;
-      HTR_PIN();
-    };
+  for (int jb = 0; jb < JB; ++jb)
 #pragma unroll
-    for (int p = 0; p < P; ++p) prefetch(buf[p], xg[p], xsg[p]);
-    const int hist = history_lane_byteaddr(lane);
-    // lane (tile tl = lane / 8, row pair q = lane % 8) holds rows 2q, 2q + 1 x the tile's 16 columns as four groups of 8
-    _Float16* dst0 = w_tile + (16 * w + 2 * (lane & 7)) * GEMM_LD + 16 * (lane >> 3);
-    auto produce = [&](StreamRegs<K>& sr, u4 (&xd)[NPT], u2& sd, int tile) {
-      DecodedStep<K> d;
-      decode_step<K>(sr, hist, d);
-      _Float16* dst = dst0 + tile * GEMM_TILE_HALVES;
-      *(h8*)dst = d.a[0];
-      *(h8*)(dst + 8) = d.a[1];
-      *(h8*)(dst + GEMM_LD) = d.a[2];
-      *(h8*)(dst + GEMM_LD + 8) = d.a[3];
+    for (int par = 0; par < 2; ++par)
 #pragma unroll
-      for (int i = 0; i < NPT; ++i) *(u4*)(x_tile + tile * GEMM_TILE_HALVES + piece_lds[i]) = xd[i];
-      if (tid < GEMM_ROWS) s_xs[tile * GEMM_ROWS + tid] = __uint_as_float(sd.x) + __uint_as_float(sd.y);
-      prefetch(sr, xd, sd);
+      for (int r = 0; r < 16; ++r) acc[jb][par][r] = 0.f;
+  float offs[JB];      // running 1534 x sum(x~) of the lane's activation rows over whole blocks (first column quarter only)
+#pragma unroll
+  for (int jb = 0; jb < JB; ++jb) offs[jb] = 0.f;
+  const float k1534 = cq == 0 ? 1534.f : 0.f;
+  // B operands: lane (activation row l32 of the 32-row block, k-group kg) reads 8 consecutive columns 16 tc + 8 kg .. + 7
+  const _Float16* b_lane = x_tile + l32 * GEMM_LD + 32 * cq + 8 * kg;
+
+  // products of one decoded step with the staged block in buffer xb
+  auto multiply = [&](const Operands& o, int xb) {
+    const _Float16* bp = b_lane + xb * GEMM_TILE_HALVES;
+#pragma unroll
+    for (int jb = 0; jb < JB; ++jb) {
+      const h8 b0 = *(const h8*)(bp + jb * 32 * GEMM_LD), b1 = *(const h8*)(bp + jb * 32 * GEMM_LD + 16);
+      acc[jb][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(o.a[0][0], b0, acc[jb][0], 0, 0, 0);
+      acc[jb][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(o.a[1][0], b0, acc[jb][1], 0, 0, 0);
+      acc[jb][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(o.a[0][1], b1, acc[jb][0], 0, 0, 0);
+      acc[jb][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(o.a[1][1], b1, acc[jb][1], 0, 0, 0);
+      offs[jb] = __builtin_fmaf(k1534, s_xs[xb * GEMM_ROWS + 32 * jb + l32], offs[jb]);
+    }
+  };
+  Operands cur;
+  auto decode_next = [&](StreamRegs<K>& sr) {
+    DecodedStep<K> d;
+    decode_step<K>(sr, hist, d);
+    prefetch(sr);
+    form(d, cur);
+  };
+
+  // ---- A step is two halves with a barrier behind each.  The two waves that share a SIMD work in opposite halves: waves
+  // 0..3 multiply block v in the first half and decode block v + 1 in the second, waves 4..7 decode block v in the
+  // first half and multiply it in the second.  So in every half each SIMD has one wave on the matrix unit and one on
+  // the vector unit, and the two run side by side (matrix instructions of one wave do not hold up the vector
+  // instructions of another).  Block v's activations are in buffer v % 3, stored during step v - 1; block v + 1's go
+  // from registers to their buffer during step v, when block v + 2 is requested.
+  // (Two copies of the loop, chosen once per wave: with the choice inside the loop the compiler keeps the registers of
+  // both kinds of half alive side by side and spills.)
+  static_assert(P == 2 || P == 4, "stream buffers rotate with the unrolled loop");
+  auto run = [&](auto lag_c) {
+    constexpr bool LAG = decltype(lag_c)::value;
+    if constexpr (!LAG) decode_next(buf[0]);
+    stage_store(0, 0);                                           // block 0 (set 0) to buffer 0; block 2 requested into set 0
+    stage_load(c_begin + 2, 0);
+    __syncthreads();
+    int xb = 0, vstep = 0;                                       // buffer of the step being multiplied, its index
+    auto step = [&](StreamRegs<K>& mine, StreamRegs<K>& ahead, bool more, int set) {      // set: register set of block v + 1
+      // every wave moves its pieces of block v + 1 to their buffer, and requests those of block v + 2, at the start of
+      // the half in which it multiplies: the matrix instructions queue up behind and hide it
+      const int xn = xb == GEMM_XBUFS - 1 ? 0 : xb + 1;
+      if constexpr (!LAG) { stage_store(xn, set); stage_load(c_begin + vstep + 3, set); multiply(cur, xb); } else decode_next(mine);
+      __syncthreads();
+      if constexpr (LAG) { stage_store(xn, set); stage_load(c_begin + vstep + 3, set); multiply(cur, xb); } else { if (more) decode_next(ahead); }
+      xb = xn;
+      ++vstep;
+      __syncthreads();
     };
     int v = 0;
-    for (; v + P <= nsteps; v += P) {
+    for (; v + P < nsteps; v += P) {
 #pragma unroll
-      for (int pp = 0; pp < P; ++pp) { produce(buf[pp], xg[pp], xsg[pp], pp & 1); __syncthreads(); }
+      for (int pp = 0; pp < P; ++pp) step(buf[pp], buf[(pp + 1) % P], true, (pp + 1) & 1);
     }
 #pragma unroll
     for (int pp = 0; pp < P; ++pp)
-      if (v + pp < nsteps) { produce(buf[pp], xg[pp], xsg[pp], pp & 1); __syncthreads(); }
-    __syncthreads();                                             // the consumers multiply the last block
-  } else {
-    // ---- consumer c: output rows 64 ih .. + 63 of the row block x activation rows 64 jh .. + 63 of the tile
-    const int c = w - GEMM_PRODUCERS, ih = c >> 1, jh = c & 1;
-    const int l32 = lane & 31, kg = lane >> 5;
-    // activation scale of this lane's two columns of the output (activation rows 64 jh + 32 bb + lane % 32)
-    float scl[2];
+      if (v + pp < nsteps) step(buf[pp], buf[(pp + 1) % P], v + pp + 1 < nsteps, (pp + 1) & 1);
+  };
+  if (w >= 4) run(std::true_type{}); else run(std::false_type{});
+
+  // ---- the four column quarters meet in LDS (the staged blocks are no longer needed: the loop ended with a barrier).
+  // D[i][j]: lane holds column j = lane % 32, register r row i = 8 (r / 4) + 4 (lane / 32) + r % 4 of the 32 x 32 piece, and
+  // row i of an A operand is strip 4 rh + i / 8, row pair i % 8: weight row 64 rh + 16 (r / 4) + 8 (lane / 32) + 2 (r % 4) + parity,
+  // so a lane's values for r = 4 rq .. 4 rq + 3, both parities interleaved, are 8 consecutive rows.
+  float scl[JB];
 #pragma unroll
-    for (int bb = 0; bb < 2; ++bb) {
-      const int j = 64 * jh + 32 * bb + l32;
-      scl[bb] = j < rows ? ((const HTR_GLOBAL float*)t.sc_g)[j0 + j] : 0.f;
-    }
-    f16v acc[2][2];
+  for (int jb = 0; jb < JB; ++jb) {
+    const int j = 32 * jb + l32;
+    scl[jb] = j < rows ? ((const HTR_GLOBAL float*)t.sc_g)[j0 + j] : 0.f;
+  }
 #pragma unroll
-    for (int a = 0; a < 2; ++a)
+  for (int phase = 0; phase < 2; ++phase) {
+    if ((cq >> 1) == phase) {
+      float* copy = s_fin + (cq & 1) * (GEMM_ROWS * GEMM_FIN_LD);
 #pragma unroll
-      for (int bb = 0; bb < 2; ++bb)
+      for (int jb = 0; jb < JB; ++jb) {
+        float* dst = copy + (32 * jb + l32) * GEMM_FIN_LD + 64 * rh + 8 * kg;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[a][bb][r] = 0.f;
-    float offs[2] = {0.f, 0.f};                // running 1534 x sum(x~) of this lane's two activation rows
-    // operands of the 32x32x16 instruction: lane (row or column = lane % 32, k-group kg = lane / 32) brings the 8
-    // consecutive k-values 8 kg .. + 7 of its row (weight row) or column (activation row): 16 bytes of an LDS tile row
-    const _Float16* a_lane = w_tile + (64 * ih + l32) * GEMM_LD + 8 * kg;
-    const _Float16* b_lane = x_tile + (64 * jh + l32) * GEMM_LD + 8 * kg;
-    auto multiply = [&](int tile) {
-      const _Float16* ap = a_lane + tile * GEMM_TILE_HALVES;
-      const _Float16* bp = b_lane + tile * GEMM_TILE_HALVES;
-      h8 A[2][2], B[2][2];                     // [k-slice parity][block]: the next slice is read while this one multiplies
-      A[0][0] = *(const h8*)ap; A[0][1] = *(const h8*)(ap + 32 * GEMM_LD);
-      B[0][0] = *(const h8*)bp; B[0][1] = *(const h8*)(bp + 32 * GEMM_LD);
-#pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        const int cur = ks & 1, nxt = cur ^ 1;
-        if (ks + 1 < 8) {
-          A[nxt][0] = *(const h8*)(ap + 16 * (ks + 1)); A[nxt][1] = *(const h8*)(ap + 32 * GEMM_LD + 16 * (ks + 1));
-          B[nxt][0] = *(const h8*)(bp + 16 * (ks + 1)); B[nxt][1] = *(const h8*)(bp + 32 * GEMM_LD + 16 * (ks + 1));
+        for (int rq = 0; rq < 4; ++rq) {
+          f4 lo = {(acc[jb][0][4 * rq] - offs[jb]) * scl[jb], (acc[jb][1][4 * rq] - offs[jb]) * scl[jb],
+                   (acc[jb][0][4 * rq + 1] - offs[jb]) * scl[jb], (acc[jb][1][4 * rq + 1] - offs[jb]) * scl[jb]};
+          f4 hi = {(acc[jb][0][4 * rq + 2] - offs[jb]) * scl[jb], (acc[jb][1][4 * rq + 2] - offs[jb]) * scl[jb],
+                   (acc[jb][0][4 * rq + 3] - offs[jb]) * scl[jb], (acc[jb][1][4 * rq + 3] - offs[jb]) * scl[jb]};
+          if (phase == 1) {
+            const f4 plo = *(const f4*)(dst + 16 * rq), phi = *(const f4*)(dst + 16 * rq + 4);
+            lo += plo; hi += phi;
+          }
+          *(f4*)(dst + 16 * rq) = lo;
+          *(f4*)(dst + 16 * rq + 4) = hi;
         }
-#pragma unroll
-        for (int a = 0; a < 2; ++a)
-#pragma unroll
-          for (int bb = 0; bb < 2; ++bb)
-            acc[a][bb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(A[cur][a], B[cur][bb], acc[a][bb], 0, 0, 0);
       }
-#pragma unroll
-      for (int bb = 0; bb < 2; ++bb) offs[bb] = __builtin_fmaf(1534.f, s_xs[tile * GEMM_ROWS + 64 * jh + 32 * bb + l32], offs[bb]);
-    };
-    // step it: the producers fill tile it % 2 while the block before it, in the other tile, is multiplied
-    __syncthreads();
-    for (int it = 1; it < nsteps; ++it) {
-      multiply((it - 1) & 1);
-      __syncthreads();
     }
-    multiply((nsteps - 1) & 1);
-    __syncthreads();                                             // every wave is through with the tiles: the output takes their place
-    // D[i][j]: lane holds column j = lane % 32, register r row i = 8 (r / 4) + 4 (lane / 32) + r % 4 of its 32 x 32 piece
-#pragma unroll
-    for (int a = 0; a < 2; ++a)
-#pragma unroll
-      for (int bb = 0; bb < 2; ++bb) {
-        float* dst = s_fin + (64 * jh + 32 * bb + l32) * GEMM_FIN_LD + 64 * ih + 32 * a + 4 * kg;
-#pragma unroll
-        for (int rq = 0; rq < 4; ++rq)
-          *(f4*)(dst + 8 * rq) = f4{(acc[a][bb][4 * rq] - offs[bb]) * scl[bb], (acc[a][bb][4 * rq + 1] - offs[bb]) * scl[bb],
-                                    (acc[a][bb][4 * rq + 2] - offs[bb]) * scl[bb], (acc[a][bb][4 * rq + 3] - offs[bb]) * scl[bb]};
-      }
+    __syncthreads();
+  }
+  // one copy: the output of the workgroup
+  for (int idx = threadIdx.x; idx < GEMM_ROWS * 32; idx += GEMM_THREADS) {
+    float* p0 = s_fin + (idx >> 5) * GEMM_FIN_LD + 4 * (idx & 31);
+    *(f4*)p0 += *(const f4*)(p0 + GEMM_ROWS * GEMM_FIN_LD);
   }
   __syncthreads();
 
@@ -1786,11 +1850,10 @@ __global__ __launch_bounds__(GEMM_THREADS) void k_linear_gemm(const uint32_t* __
   // in the scratch half of the workspace with device-scope stores, and ONE flag word per workgroup, set after every
   // thread's stores have completed, says it is there.  The last split (dispatched after the others, so waiting for
   // them cannot deadlock; bounded all the same) waits for the flags, adds the tiles to its own in LDS and clears the flags.
-  constexpr int WAVES = GEMM_PRODUCERS + GEMM_CONSUMERS;
+  constexpr int WAVES = WG_WAVES;
   const size_t wg0 = ((size_t)mt * gridDim.y + rb) * S;              // index of split 0's workgroup of this (row block, tile)
   uint32_t* ready = (uint32_t*)part;                                 // one word per workgroup, zero between launches
   float* tiles = t.tiles;                                            // [workgroups][128][128] floats in the scratch half of the workspace
-  uint32_t& s_failed = *(uint32_t*)(s_xs + 2 * GEMM_ROWS);       // the finisher's wait gave up (behind the sums: not overlaid by the output)
   if (S > 1) {
     typedef unsigned long long u64;
     if (s_idx != S - 1) {

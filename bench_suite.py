@@ -185,9 +185,11 @@ def moe(dev):
 
 
 def prefill(dev):
-    """dequant_w + library GEMM against fused 32-row launches, eager calls through ops (wall time of the host included)."""
+    """129 rows and more: dequant_w + library GEMM against ONE launch of the fused decode -> matrix-unit kernel (rotation
+    launch included) and against fused launches of 128 rows; eager calls, events on the launch stream."""
+    L = _native.lib()
     out = []
-    for (m, n) in ((4096, 4096), (14336, 4096), (4096, 14336)):
+    for (m, n) in ((4096, 4096), (6144, 4096), (14336, 4096), (4096, 14336)):
         w = wire.synth_linear(m, n, 4, SEED + 11, dev)
 
         def eager(fn, reps=20):
@@ -200,16 +202,28 @@ def prefill(dev):
         W = ops.dequant_w(*w)
         row = {"m": m, "n": n, "K": 4, "dequant_w_us": round(td, 1),
                "dequant_w_written_GBps": round(2.0 * m * n / td / 1e3, 1), "rows": []}
-        for M in (32, 64, 128, 256, 512):
+        for M in (64, 128, 160, 192, 256, 384, 512):
             x = wire.synth_activation(M, n, SEED + 3, torch.bfloat16, dev)
+            y = torch.empty(M, m, dtype=torch.bfloat16, device=dev)
             tg = eager(lambda: torch.nn.functional.linear(x, W))
-            old, ops.GEMV_LOOP_MAX = ops.GEMV_LOOP_MAX, 10 ** 9
-            try:
-                tl = eager(lambda: ops.linear(x, *w), reps=5)
-            finally:
-                ops.GEMV_LOOP_MAX = old
-            row["rows"].append({"M": M, "gemm_us": round(tg, 1), "dequant_plus_gemm_us": round(td + tg, 1),
-                                "fused_launches_us": round(tl, 1)})
+            ws = torch.zeros(L.htr_workspace_bytes(m, n, 4, M, 0), dtype=torch.uint8, device=dev)
+
+            def one_launch():
+                _native.check(L.htr_linear(w[0].data_ptr(), w[1].data_ptr(), w[2].data_ptr(), w[3].data_ptr(), x.data_ptr(), None,
+                                           y.data_ptr(), m, n, 4, M, _native.BF16, _native.BF16, 0, ws.data_ptr(), ws.numel(),
+                                           torch.cuda.current_stream().cuda_stream))
+
+            t1 = eager(one_launch)
+            rec = {"M": M, "gemm_us": round(tg, 1), "dequant_plus_gemm_us": round(td + tg, 1), "one_fused_launch_us": round(t1, 1),
+                   "ops_takes_fused": M <= ops.fused_max_rows(m, n)}
+            if M > 128:
+                old_max, old_rows = ops.GEMV_LOOP_MAX, ops.LAUNCH_MAX_M
+                ops.GEMV_LOOP_MAX, ops.LAUNCH_MAX_M = 10 ** 9, 128
+                try:
+                    rec["launches_of_128_rows_us"] = round(eager(lambda: ops.linear(x, *w), reps=5), 1)
+                finally:
+                    ops.GEMV_LOOP_MAX, ops.LAUNCH_MAX_M = old_max, old_rows
+            row["rows"].append(rec)
         out.append(row)
     return out
 

@@ -2622,8 +2622,8 @@ inline bool make_batch_plan(int m, int n, int M, int want_S, BatchPlan& bp) {
   return found;
 }
 
-// ---- GEMM kernel (more than 128 rows): tiles of 128 activation rows in the grid's z, split S of the column blocks while the
-// grid stays within one workgroup per compute unit (its 137 KB of LDS leave room for one)
+// ---- GEMM kernel (more than 128 rows): tiles of GEMM_ROWS activation rows in the grid's z, split S of the column blocks
+// while the grid stays within one workgroup per compute unit (256 registers per lane leave room for one)
 struct GemmPlan { int S, cb, mtiles, wgs; };
 constexpr int GEMM_MIN_M = HTR_MAX_ROWS_PER_TILE + 1;       // rows from which the library policy takes the GEMM kernel
 inline bool make_gemm_plan(int m, int n, int M, int want_S, GemmPlan& gp) {

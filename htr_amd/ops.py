@@ -21,12 +21,29 @@ LAUNCH_MAX_M = max(1, min(_native.MAX_BATCH, int(os.environ.get("HTR_GEMV_MAX_M"
 GROUP_MAX_M = _native.MAX_GROUP_ROWS      # rows per entry of a grouped launch
 # explicit chunk length (steps per workgroup) for experiments; 0 = library policy
 NSPLIT = int(os.environ.get("HTR_NSPLIT", "0"))
-# Above this many activation rows the weight is dequantized once to the original basis (bf16) and a library GEMM does
-# the product, as the reference does for prefill (HTR_PREFILL="w", htr/ops.py:52-54,89-93); up to it, the fused
-# decode kernel runs in launches of LAUNCH_MAX_M rows (the reference's HTR_GEMV_LOOP_MAX, htr/ops.py:59-61).
-# Measured on MI355X (K4): one fused launch of 128 rows takes 32 / 42 / 59 us on 4096x4096 / 14336x4096 / 4096x14336,
-# dequantize + GEMM 42 / 73 / 105 us; two fused launches (256 rows) no longer beat it.
-GEMV_LOOP_MAX = int(os.environ.get("HTR_GEMV_LOOP_MAX", "128"))
+# Above a number of activation rows the weight is dequantized once to the original basis (bf16) and a library GEMM does
+# the product, as the reference does for prefill (HTR_PREFILL="w", htr/ops.py:52-54,89-93); up to it, fused launches of
+# LAUNCH_MAX_M rows run (the reference's HTR_GEMV_LOOP_MAX, htr/ops.py:59-61).  Up to 128 rows that is the batched decode
+# kernel; beyond, the fused decode -> matrix-unit kernel, which re-decodes the weight once per 96 activation rows and so
+# only pays while few such tiles cover the input.  Measured on MI355X (K4, rotation launch included, against
+# dequantize + GEMM): 14336x4096 47 us at 160..192 rows (1.7x), 82..90 us at 256..384 rows (1.0..1.1x), slower from 512;
+# 28672x4096 1.5x at 160..192 rows, 1.2x at 256..288; 4096x14336 1.7..1.8x up to 192 rows, 1.1..1.25x up to 384;
+# 6144x4096 1.05..1.4x up to 384; 4096x4096 never (0.75..0.98x).  HTR_GEMV_LOOP_MAX overrides the limit for every shape.
+_LOOP_MAX_ENV = os.environ.get("HTR_GEMV_LOOP_MAX")
+GEMV_LOOP_MAX = None if _LOOP_MAX_ENV is None else int(_LOOP_MAX_ENV)
+
+
+def fused_max_rows(m, n):
+    """Activation rows up to which the fused kernels take an [m, n] linear; more rows go to dequantize + library GEMM."""
+    if GEMV_LOOP_MAX is not None:
+        return GEMV_LOOP_MAX
+    if n >= 8192:
+        return 384
+    if m * n >= 6144 * 4096:
+        return 192 if m >= 8192 else 384
+    return 128
+
+
 # How inputs beyond GEMV_LOOP_MAX rows are multiplied (the reference's HTR_PREFILL, htr/ops.py:52-54): "w" = dequantize
 # to the original basis and one library GEMM (default); "rot" = stay in the rotated basis: rotate the activations, GEMM
 # against the dequantized Q, rotate the result (the reference's slower first-version path, htr/ops.py:101-104; here
@@ -204,13 +221,14 @@ def _linear_impl(x2, qweight, scales, su, sv, bias, out_dtype=None):
             raise RuntimeError("HTR-W1 tensors must be contiguous and on the device of x")
     if bias is not None and (bias.dtype != out_dtype or bias.numel() != m or bias.device != x2.device):
         raise RuntimeError("bias must be [m] in the output dtype on the device of x")
-    if M > GEMV_LOOP_MAX and PREFILL == "rot":
+    loop_max = fused_max_rows(m, n)
+    if M > loop_max and PREFILL == "rot":
         xr = wire.blk_had_cols_T(x2.float() * wire.unpack_signs(su, n).to(x2.device))
         yr = wire.blk_had_cols_T(xr @ dequant_q(qweight, scales).T) * wire.unpack_signs(sv, m).to(x2.device)
         if bias is not None:
             yr = yr + bias.float()
         return yr.to(out_dtype)
-    if M > GEMV_LOOP_MAX:
+    if M > loop_max:
         if PREFILL != "w":
             raise RuntimeError(f"HTR_PREFILL = {PREFILL!r}: expected 'w' or 'rot'")
         W = dequant_w(qweight, scales, su, sv)

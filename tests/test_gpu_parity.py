@@ -98,7 +98,7 @@ def test_prefill_path_dequant_then_gemm(dev, oracle):
     print("prefill M=160", flush=True)
     qw, sc, su, sv, x = _case(512, 384, 4, 160, 808)
     bias = torch.randn(512, generator=torch.Generator().manual_seed(2)).bfloat16()
-    assert 160 > ops.GEMV_LOOP_MAX
+    assert 160 > ops.fused_max_rows(512, 384)
     y = ops.linear(x.to(dev), *[t.to(dev) for t in (qw, sc, su, sv)], bias.to(dev))
     assert y.dtype == torch.bfloat16 and tuple(y.shape) == (160, 512)
     ref = _ref(oracle, qw, sc, su, sv, x, bias)
@@ -356,6 +356,83 @@ def test_small_batch_gemm_shapes(dev, oracle, K, M, m, n, monkeypatch):
     ref = _ref(oracle, qw, sc, su, sv, x)
     for r in range(M):
         assert _rel(y[r], ref[r]) <= REL_TOL, (r, _rel(y[r], ref[r]))
+
+
+# ---- more than 128 activation rows in one launch: the fused decode -> matrix-unit kernel.  Row counts on both sides of
+# the 96-row tiles, every K, explicit column splits (nsplit = 2^28 + S) including the exchange between splits, bias and
+# all three output types, and a second call on the same workspace (the flags must be back at zero).
+_GEMM = [(4, 130, 256, 512, 0), (4, 200, 256, 512, 2), (4, 256, 384, 1024, 4), (4, 300, 256, 512, 1), (4, 257, 1024, 2048, 0),
+         (2, 129, 256, 384, 0), (3, 192, 384, 512, 2), (5, 193, 256, 512, 0), (6, 150, 256, 256, 1), (7, 288, 128, 384, 3),
+         (8, 161, 256, 512, 0), (4, 1000, 256, 256, 0), (4, 2048, 128, 256, 1), (4, 96, 256, 512, 1), (4, 40, 256, 384, 2)]
+
+
+@pytest.mark.parametrize("K,M,m,n,S", _GEMM)
+def test_more_than_128_rows_in_one_launch(dev, oracle, K, M, m, n, S):
+    import ctypes
+    from htr_amd import _native
+    print(f"gemm kernel K={K} M={M} {m}x{n} S={S}", flush=True)
+    L = _native.lib()
+    nsplit = (1 << 28) | S if (S or M <= 128) else 0
+    qw, sc, su, sv, x = _case(m, n, K, M, 9000 + 17 * K + M)
+    d = [t.to(dev) for t in (qw, sc, su, sv)]
+    xd = x.to(dev)
+    plan = (ctypes.c_int * 6)()
+    assert L.htr_linear_plan(m, n, K, M, nsplit, plan) == 0
+    assert plan[2] == (M + 95) // 96 and plan[1] == plan[3] * (m // 128) * plan[2]       # row tiles; splits x row blocks x tiles
+    if S:
+        assert plan[3] == S
+    need = L.htr_workspace_bytes(m, n, K, M, nsplit)
+    assert need > 0
+    ws = torch.zeros(need, dtype=torch.uint8, device=dev)
+    y = torch.full((M, m), float("nan"), dtype=torch.float32, device=dev)
+    st = torch.cuda.current_stream().cuda_stream
+
+    def call():
+        _native.check(L.htr_linear(d[0].data_ptr(), d[1].data_ptr(), d[2].data_ptr(), d[3].data_ptr(), xd.data_ptr(), None,
+                                   y.data_ptr(), m, n, K, M, _native.BF16, _native.F32, nsplit, ws.data_ptr(), ws.numel(), st))
+        torch.cuda.synchronize()
+
+    call()
+    first = y.clone()
+    ref = _ref(oracle, qw, sc, su, sv, x)
+    got = first.cpu().numpy()
+    for r in (0, 95, 96, M // 2, M - 1):
+        if r < M:
+            assert _rel(got[r], ref[r]) <= REL_TOL, (r, _rel(got[r], ref[r]))
+    assert _rel(got, ref) <= REL_TOL
+    y.fill_(float("nan"))
+    call()
+    assert torch.equal(first, y)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_more_than_128_rows_through_ops_with_bias(dev, oracle, dtype, monkeypatch):
+    from htr_amd import ops
+    print(f"gemm kernel through ops, {dtype}", flush=True)
+    monkeypatch.setattr(ops, "GEMV_LOOP_MAX", 1 << 30)
+    qw, sc, su, sv, x = _case(384, 512, 4, 210, 9100, dtype)
+    bias = torch.randn(384, generator=torch.Generator().manual_seed(9)).to(dtype)
+    y = ops.linear(x.to(dev), *[t.to(dev) for t in (qw, sc, su, sv)], bias.to(dev))
+    assert y.dtype == dtype and tuple(y.shape) == (210, 384)
+    ref = _ref(oracle, qw, sc, su, sv, x, bias)
+    tol = REL_TOL if dtype == torch.float32 else 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -9
+    assert _rel(y.float().cpu().numpy(), ref) <= tol
+
+
+def test_fused_row_limit_follows_the_shape(dev, oracle):
+    """ops.linear takes the fused kernels up to a row count that depends on the shape, and dequantize + GEMM beyond;
+    both sides of the switch give the same product."""
+    from htr_amd import ops
+    assert ops.fused_max_rows(4096, 4096) == 128 and ops.fused_max_rows(14336, 4096) == 192
+    assert ops.fused_max_rows(4096, 14336) == 384 and ops.fused_max_rows(6144, 4096) == 384
+    print("gemm kernel at the policy's shape", flush=True)
+    qw, sc, su, sv, x = _case(14336, 4096, 4, 192, 9200)
+    d = [t.to(dev) for t in (qw, sc, su, sv)]
+    y = ops.linear_f32out(x.to(dev), *d).cpu().numpy()
+    ref = _ref(oracle, qw, sc, su, sv, x)
+    assert _rel(y, ref) <= REL_TOL
+    y2 = ops.linear(torch.cat([x, x[:8]]).to(dev), *d).float().cpu().numpy()          # 200 rows: the prefill path
+    assert _rel(y2[:192], ref) <= 2.0 ** -6
 
 
 def test_moe_expert_stack_top6_of_64(dev, oracle):

@@ -50,6 +50,7 @@ def test_constants(L, oracle):
 
 
 def test_validation_codes_without_gpu(L):
+    from htr_amd import _native
     p = ctypes.c_void_p(0x1000)                # never dereferenced: every case below fails validation first
     ok_ws = ctypes.c_void_p(0x100000)
     call = lambda **kw: L.htr_linear(kw.get("qw", p), p, p, p, p, None, kw.get("y", p), kw.get("m", 256), kw.get("n", 256),
@@ -58,8 +59,9 @@ def test_validation_codes_without_gpu(L):
     assert call(qw=None) == 1
     assert call(K=1) == 2 and call(K=9) == 2
     assert call(m=200) == 3 and call(n=0) == 3
-    assert call(M=0) == 4 and call(M=129) == 4
+    assert call(M=0) == 4 and call(M=_native.MAX_BATCH + 1) == 4
     assert call(M=33, ns=4) == 4               # an explicit chunked plan stops at 32 rows
+    assert call(M=129, ns=(1 << 29) | 1) == 4  # an explicit batched plan at 128
     assert call(xd=3) == 5 and call(yd=-1) == 5
     assert call(ws=None) == 6 and call(wsb=16) == 6 and call(ws=ctypes.c_void_p(0x100010)) == 6
     assert call(qw=ctypes.c_void_p(0x1004)) == 7
@@ -106,6 +108,28 @@ def test_launch_plan_is_consistent(L, m, n, M):
     assert L.htr_linear_plan(m, n, 4, M, 1, out) == 0
     if out[0] == 1:
         assert out[1] == rbs * nblk
+
+
+@pytest.mark.parametrize("m,n", [(128, 128), (4096, 4096), (14336, 4096), (4096, 14336), (28672, 4096)])
+@pytest.mark.parametrize("M", [129, 192, 193, 384, 1000, 2048])
+def test_plan_for_more_than_128_rows(L, m, n, M):
+    """The fused decode -> matrix-unit kernel: tiles of 96 activation rows, up to 8 column splits while the grid stays within
+    the compute units, no empty split; the workspace holds the rotated activations and, with splits, a tile per workgroup."""
+    out = (ctypes.c_int * 6)()
+    assert L.htr_linear_plan(m, n, 4, M, 0, out) == 0
+    cb, wgs, tiles, S, prerot, lds = list(out)
+    nblk, rbs = n // 128, m // 128
+    assert tiles == -(-M // 96) and wgs == S * rbs * tiles and prerot == 1 and lds <= 160 * 1024
+    assert 1 <= S <= 8 and S == -(-nblk // cb) and (S == 1 or wgs <= 256)
+    need = L.htr_workspace_bytes(m, n, 4, M, 0)
+    assert need >= 256 + M * n * 2 + (wgs * 96 * 128 * 4 if S > 1 else 0)
+    for want in (1, 2, 8):
+        if want > nblk or -(-nblk // -(-nblk // want)) != want:
+            assert L.htr_linear_plan(m, n, 4, M, (1 << 28) | want, out) != 0        # such a split would leave one empty
+            continue
+        assert L.htr_linear_plan(m, n, 4, M, (1 << 28) | want, out) == 0 and out[3] == want and out[1] == want * rbs * tiles
+    # bit 28 takes the kernel below its policy's row count too
+    assert L.htr_linear_plan(m, n, 4, 40, (1 << 28) | 1, out) == 0 and out[2] == 1 and out[1] == rbs
 
 
 @pytest.mark.parametrize("cus", [32, 64, 120, 256, 304])

@@ -215,7 +215,7 @@ def prefill(dev):
 
             t1 = eager(one_launch)
             rec = {"M": M, "gemm_us": round(tg, 1), "dequant_plus_gemm_us": round(td + tg, 1), "one_fused_launch_us": round(t1, 1),
-                   "ops_takes_fused": M <= ops.fused_max_rows(m, n)}
+                   "ops_rows_per_fused_launch": ops.fused_rows_per_launch(m, n, M)}       # 0: ops.linear dequantizes
             if M > 128:
                 old_max, old_rows = ops.GEMV_LOOP_MAX, ops.LAUNCH_MAX_M
                 ops.GEMV_LOOP_MAX, ops.LAUNCH_MAX_M = 10 ** 9, 128

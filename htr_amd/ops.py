@@ -22,26 +22,46 @@ GROUP_MAX_M = _native.MAX_GROUP_ROWS      # rows per entry of a grouped launch
 # explicit chunk length (steps per workgroup) for experiments; 0 = library policy
 NSPLIT = int(os.environ.get("HTR_NSPLIT", "0"))
 # Above a number of activation rows the weight is dequantized once to the original basis (bf16) and a library GEMM does
-# the product, as the reference does for prefill (HTR_PREFILL="w", htr/ops.py:52-54,89-93); up to it, fused launches of
-# LAUNCH_MAX_M rows run (the reference's HTR_GEMV_LOOP_MAX, htr/ops.py:59-61).  Up to 128 rows that is the batched decode
-# kernel; beyond, the fused decode -> matrix-unit kernel, which re-decodes the weight once per 96 activation rows and so
-# only pays while few such tiles cover the input.  Measured on MI355X (K4, rotation launch included, against
-# dequantize + GEMM): 14336x4096 47 us at 160..192 rows (1.7x), 82..90 us at 256..384 rows (1.0..1.1x), slower from 512;
-# 28672x4096 1.5x at 160..192 rows, 1.2x at 256..288; 4096x14336 1.7..1.8x up to 192 rows, 1.1..1.25x up to 384;
-# 6144x4096 1.05..1.4x up to 384; 4096x4096 never (0.75..0.98x).  HTR_GEMV_LOOP_MAX overrides the limit for every shape.
+# the product, as the reference does for prefill (HTR_PREFILL="w", htr/ops.py:52-54,89-93); up to it, fused launches
+# run (the reference's HTR_GEMV_LOOP_MAX, htr/ops.py:59-61): up to 128 rows the batched decode kernel; beyond, either the
+# fused decode -> matrix-unit kernel in ONE launch (it re-decodes the weight once per 96 activation rows, so it pays while
+# few such tiles cover the input and the grid stays within the chip) or launches of 128 rows, whichever was faster.
+# Measured on MI355X (K4, eager, us; one fused launch incl. its rotation launch / launches of 128 rows / dequantize + GEMM):
+#   14336x4096: 160 rows 46 / 62 / 77, 192 rows 48 / 69 / 81, 256 rows 85 / 79 / 89, 384 rows 99 / 128 / 96
+#   4096x14336: 160 rows 67 / 64 / 116, 192 rows 70 / 67 / 126, 256 rows 95 / 82 / 94, 384 rows 110 / 124 / 114
+#   6144x4096:  160 rows 46 / 43 / 48, 192 rows 48 / 51 / 51, 256 rows 44 / 57 / 60, 384 rows 49 / 84 / 54, 512 rows 85 / 108 / 56
+#   4096x4096:  160 rows 45 / 36 / 41, 256 rows 48 / 48 / 37, 512 rows 49 / 90 / 44
+# HTR_GEMV_LOOP_MAX overrides the row limit for every shape (launches of LAUNCH_MAX_M rows up to it).
 _LOOP_MAX_ENV = os.environ.get("HTR_GEMV_LOOP_MAX")
 GEMV_LOOP_MAX = None if _LOOP_MAX_ENV is None else int(_LOOP_MAX_ENV)
+ONE_LAUNCH = _native.MAX_BATCH
+
+
+def fused_rows_per_launch(m, n, M):
+    """Rows per fused launch for M activation rows on an [m, n] linear; 0 = dequantize + library GEMM."""
+    if GEMV_LOOP_MAX is not None:
+        return LAUNCH_MAX_M if M <= GEMV_LOOP_MAX else 0
+    rows = 0
+    if M <= _native.MAX_ROWS_PER_TILE:
+        rows = _native.MAX_ROWS_PER_TILE
+    elif m * n < 6144 * 4096:
+        rows = 0
+    elif n >= 8192 or m >= 8192:
+        # long rows: the fused GEMM kernel needs column splits and their exchange, two batched launches are ahead;
+        # many row blocks: two tiles of 96 rows fill the chip once
+        rows = ONE_LAUNCH if (n < 8192 and M <= 192) else (_native.MAX_ROWS_PER_TILE if M <= 256 else 0)
+    else:
+        rows = ONE_LAUNCH if M <= 384 else 0
+    return min(rows, LAUNCH_MAX_M)
 
 
 def fused_max_rows(m, n):
     """Activation rows up to which the fused kernels take an [m, n] linear; more rows go to dequantize + library GEMM."""
     if GEMV_LOOP_MAX is not None:
         return GEMV_LOOP_MAX
-    if n >= 8192:
-        return 384
-    if m * n >= 6144 * 4096:
-        return 192 if m >= 8192 else 384
-    return 128
+    if m * n < 6144 * 4096:
+        return _native.MAX_ROWS_PER_TILE
+    return 256 if (n >= 8192 or m >= 8192) else 384
 
 
 # How inputs beyond GEMV_LOOP_MAX rows are multiplied (the reference's HTR_PREFILL, htr/ops.py:52-54): "w" = dequantize
@@ -221,14 +241,14 @@ def _linear_impl(x2, qweight, scales, su, sv, bias, out_dtype=None):
             raise RuntimeError("HTR-W1 tensors must be contiguous and on the device of x")
     if bias is not None and (bias.dtype != out_dtype or bias.numel() != m or bias.device != x2.device):
         raise RuntimeError("bias must be [m] in the output dtype on the device of x")
-    loop_max = fused_max_rows(m, n)
-    if M > loop_max and PREFILL == "rot":
+    per_launch = fused_rows_per_launch(m, n, M)
+    if per_launch == 0 and PREFILL == "rot":
         xr = wire.blk_had_cols_T(x2.float() * wire.unpack_signs(su, n).to(x2.device))
         yr = wire.blk_had_cols_T(xr @ dequant_q(qweight, scales).T) * wire.unpack_signs(sv, m).to(x2.device)
         if bias is not None:
             yr = yr + bias.float()
         return yr.to(out_dtype)
-    if M > loop_max:
+    if per_launch == 0:
         if PREFILL != "w":
             raise RuntimeError(f"HTR_PREFILL = {PREFILL!r}: expected 'w' or 'rot'")
         W = dequant_w(qweight, scales, su, sv)
@@ -239,8 +259,8 @@ def _linear_impl(x2, qweight, scales, su, sv, bias, out_dtype=None):
     y = torch.empty((M, m), dtype=out_dtype, device=x2.device)
     code = _DTYPE_CODE[out_dtype]
     with torch.cuda.device(x2.device):
-        for r0 in range(0, M, LAUNCH_MAX_M):
-            r1 = min(M, r0 + LAUNCH_MAX_M)
+        for r0 in range(0, M, per_launch):
+            r1 = min(M, r0 + per_launch)
             _launch(x2[r0:r1], qweight, scales, su, sv, bias, y[r0:r1], m, n, K, code)
     return y
 

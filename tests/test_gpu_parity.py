@@ -420,19 +420,27 @@ def test_more_than_128_rows_through_ops_with_bias(dev, oracle, dtype, monkeypatc
 
 
 def test_fused_row_limit_follows_the_shape(dev, oracle):
-    """ops.linear takes the fused kernels up to a row count that depends on the shape, and dequantize + GEMM beyond;
-    both sides of the switch give the same product."""
+    """ops.linear takes one launch of the fused GEMM kernel, launches of 128 rows or dequantize + GEMM depending on shape
+    and row count; all three give the same product."""
     from htr_amd import ops
-    assert ops.fused_max_rows(4096, 4096) == 128 and ops.fused_max_rows(14336, 4096) == 192
-    assert ops.fused_max_rows(4096, 14336) == 384 and ops.fused_max_rows(6144, 4096) == 384
+    big = ops.ONE_LAUNCH
+    assert ops.fused_max_rows(4096, 4096) == 128 and ops.fused_max_rows(14336, 4096) == 256
+    assert ops.fused_max_rows(4096, 14336) == 256 and ops.fused_max_rows(6144, 4096) == 384
+    assert [ops.fused_rows_per_launch(14336, 4096, M) for M in (1, 128, 129, 192, 193, 256, 257)] == [128, 128, big, big, 128, 128, 0]
+    assert [ops.fused_rows_per_launch(4096, 14336, M) for M in (129, 256, 257)] == [128, 128, 0]
+    assert [ops.fused_rows_per_launch(6144, 4096, M) for M in (129, 384, 385)] == [big, big, 0]
+    assert ops.fused_rows_per_launch(4096, 4096, 129) == 0
     print("gemm kernel at the policy's shape", flush=True)
     qw, sc, su, sv, x = _case(14336, 4096, 4, 192, 9200)
     d = [t.to(dev) for t in (qw, sc, su, sv)]
-    y = ops.linear_f32out(x.to(dev), *d).cpu().numpy()
     ref = _ref(oracle, qw, sc, su, sv, x)
+    y = ops.linear_f32out(x.to(dev), *d).cpu().numpy()                                # one launch of the GEMM kernel
     assert _rel(y, ref) <= REL_TOL
-    y2 = ops.linear(torch.cat([x, x[:8]]).to(dev), *d).float().cpu().numpy()          # 200 rows: the prefill path
-    assert _rel(y2[:192], ref) <= 2.0 ** -6
+    x200 = torch.cat([x, x[:8]])
+    y2 = ops.linear_f32out(x200.to(dev), *d).cpu().numpy()                            # 128 + 72 rows, batched kernel
+    assert _rel(y2[:192], ref) <= REL_TOL and _rel(y2[192:], ref[:8]) <= REL_TOL
+    y3 = ops.linear(torch.cat([x, x[:100]]).to(dev), *d).float().cpu().numpy()        # 292 rows: dequantize + GEMM
+    assert _rel(y3[:192], ref) <= 2.0 ** -6
 
 
 def test_moe_expert_stack_top6_of_64(dev, oracle):

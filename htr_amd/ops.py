@@ -27,31 +27,33 @@ NSPLIT = int(os.environ.get("HTR_NSPLIT", "0"))
 # fused decode -> matrix-unit kernel in ONE launch (it re-decodes the weight once per 96 activation rows, so it pays while
 # few such tiles cover the input and the grid stays within the chip) or launches of 128 rows, whichever was faster.
 # Measured on MI355X (K4, eager, us; one fused launch incl. its rotation launch / launches of 128 rows / dequantize + GEMM):
-#   14336x4096: 160 rows 46 / 62 / 77, 192 rows 48 / 69 / 81, 256 rows 85 / 79 / 89, 384 rows 99 / 128 / 96
-#   4096x14336: 160 rows 67 / 64 / 116, 192 rows 70 / 67 / 126, 256 rows 95 / 82 / 94, 384 rows 110 / 124 / 114
-#   6144x4096:  160 rows 46 / 43 / 48, 192 rows 48 / 51 / 51, 256 rows 44 / 57 / 60, 384 rows 49 / 84 / 54, 512 rows 85 / 108 / 56
-#   4096x4096:  160 rows 45 / 36 / 41, 256 rows 48 / 48 / 37, 512 rows 49 / 90 / 44
-# HTR_GEMV_LOOP_MAX overrides the row limit for every shape (launches of LAUNCH_MAX_M rows up to it).
+#   14336x4096: 160 rows 47 / 63 / 77, 192 rows 50 / 73 / 81, 256 rows 87 / 81 / 90, 384 rows 98 / 129 / 97
+#   4096x14336: 160 rows 52 / 61 / 117, 192 rows 55 / 68 / 127, 256 rows 89 / 88 / 96, 384 rows 95 / 133 / 117, 512 rows 147 / 162 / 129
+#   6144x4096:  160 rows 35 / 46 / 48, 192 rows 37 / 50 / 51, 256 rows 45 / 58 / 59, 384 rows 49 / 83 / 53, 512 rows 87 / 109 / 56
+#   4096x4096:  160 rows 32 / 37 / 41, 192 rows 33 / 51 / 44, 256 rows 37 / 46 / 37, 384 rows 41 / 69 / 40, 512 rows 49 / 90 / 45
+# So: one fused launch while its tiles x the weight's row blocks fit the chip in one round, up to 384 rows (192 on a
+# matrix as small as 4096x4096, whose dequantization is cheap); two launches of 128 rows where a third tile would start
+# a second round (14336x4096 at 193..256 rows); else dequantize.  HTR_GEMV_LOOP_MAX overrides the row limit for every
+# shape (launches of LAUNCH_MAX_M rows up to it).
 _LOOP_MAX_ENV = os.environ.get("HTR_GEMV_LOOP_MAX")
 GEMV_LOOP_MAX = None if _LOOP_MAX_ENV is None else int(_LOOP_MAX_ENV)
 ONE_LAUNCH = _native.MAX_BATCH
+_TILE_ROWS = 96          # activation rows per tile of the fused GEMM kernel
+_CHIP_WORKGROUPS = 256   # one workgroup per compute unit of the MI355X the table above was measured on
 
 
 def fused_rows_per_launch(m, n, M):
     """Rows per fused launch for M activation rows on an [m, n] linear; 0 = dequantize + library GEMM."""
     if GEMV_LOOP_MAX is not None:
         return LAUNCH_MAX_M if M <= GEMV_LOOP_MAX else 0
-    rows = 0
     if M <= _native.MAX_ROWS_PER_TILE:
         rows = _native.MAX_ROWS_PER_TILE
     elif m * n < 6144 * 4096:
-        rows = 0
-    elif n >= 8192 or m >= 8192:
-        # long rows: the fused GEMM kernel needs column splits and their exchange, two batched launches are ahead;
-        # many row blocks: two tiles of 96 rows fill the chip once
-        rows = ONE_LAUNCH if (n < 8192 and M <= 192) else (_native.MAX_ROWS_PER_TILE if M <= 256 else 0)
+        rows = ONE_LAUNCH if (m * n >= 4096 * 4096 and M <= 192) else 0
+    elif M <= 384 and (m // 128) * -(-M // _TILE_ROWS) <= _CHIP_WORKGROUPS:
+        rows = ONE_LAUNCH
     else:
-        rows = ONE_LAUNCH if M <= 384 else 0
+        rows = _native.MAX_ROWS_PER_TILE if M <= 256 else 0
     return min(rows, LAUNCH_MAX_M)
 
 
@@ -60,8 +62,8 @@ def fused_max_rows(m, n):
     if GEMV_LOOP_MAX is not None:
         return GEMV_LOOP_MAX
     if m * n < 6144 * 4096:
-        return _native.MAX_ROWS_PER_TILE
-    return 256 if (n >= 8192 or m >= 8192) else 384
+        return 192 if m * n >= 4096 * 4096 else _native.MAX_ROWS_PER_TILE
+    return 384 if (m // 128) * 4 <= _CHIP_WORKGROUPS else 256
 
 
 # How inputs beyond GEMV_LOOP_MAX rows are multiplied (the reference's HTR_PREFILL, htr/ops.py:52-54): "w" = dequantize

@@ -424,12 +424,13 @@ def test_fused_row_limit_follows_the_shape(dev, oracle):
     and row count; all three give the same product."""
     from htr_amd import ops
     big = ops.ONE_LAUNCH
-    assert ops.fused_max_rows(4096, 4096) == 128 and ops.fused_max_rows(14336, 4096) == 256
-    assert ops.fused_max_rows(4096, 14336) == 256 and ops.fused_max_rows(6144, 4096) == 384
+    assert ops.fused_max_rows(4096, 4096) == 192 and ops.fused_max_rows(14336, 4096) == 256 and ops.fused_max_rows(1024, 4096) == 128
+    assert ops.fused_max_rows(4096, 14336) == 384 and ops.fused_max_rows(6144, 4096) == 384
     assert [ops.fused_rows_per_launch(14336, 4096, M) for M in (1, 128, 129, 192, 193, 256, 257)] == [128, 128, big, big, 128, 128, 0]
-    assert [ops.fused_rows_per_launch(4096, 14336, M) for M in (129, 256, 257)] == [128, 128, 0]
+    assert [ops.fused_rows_per_launch(4096, 14336, M) for M in (129, 384, 385)] == [big, big, 0]
     assert [ops.fused_rows_per_launch(6144, 4096, M) for M in (129, 384, 385)] == [big, big, 0]
-    assert ops.fused_rows_per_launch(4096, 4096, 129) == 0
+    assert [ops.fused_rows_per_launch(4096, 4096, M) for M in (129, 192, 193)] == [big, big, 0]
+    assert ops.fused_rows_per_launch(2048, 2048, 129) == 0
     print("gemm kernel at the policy's shape", flush=True)
     qw, sc, su, sv, x = _case(14336, 4096, 4, 192, 9200)
     d = [t.to(dev) for t in (qw, sc, su, sv)]

@@ -1710,23 +1710,17 @@ __global__ __launch_bounds__(GEMM_THREADS) void k_linear_gemm(const uint32_t* __
   for (int p = 0; p < P; ++p) prefetch(buf[p]);
   const int hist = history_lane_byteaddr(lane);
 
-  // A operands of one step, after the swap: [even | odd rows][tile column 2 cq | 2 cq + 1]
+  // A operands of one step: [even | odd rows][columns 0..7 | 8..15 of the lane's tile].  The matrix instruction sums over
+  // 16 k-slots, lanes 0..31 bringing slots 0..7 and lanes 32..63 slots 8..15 of row lane % 32; which weight columns the
+  // slots stand for is free as long as the B operand agrees.  So the decode registers are used as they are: in the
+  // first instruction of a pair the slots are columns 0..7 of tile column 2 cq (lower lanes) and columns 0..7 of tile
+  // column 2 cq + 1 (upper lanes), in the second columns 8..15 of both, and the B operand reads the activations of
+  // exactly those columns.  No lane exchange.
   struct Operands { h8 a[2][2]; };
   auto form = [&](const DecodedStep<K>& d, Operands& o) {
     // d.a[0], d.a[1] = row 2q columns 0..7, 8..15; d.a[2], d.a[3] = row 2q + 1 columns 0..7, 8..15 of the lane's tile
 #pragma unroll
-    for (int par = 0; par < 2; ++par) {
-      const u4 lo = __builtin_bit_cast(u4, d.a[2 * par]), hi = __builtin_bit_cast(u4, d.a[2 * par + 1]);
-      u4 t0, t1;
-#pragma unroll
-      for (int dw = 0; dw < 4; ++dw) {
-        // x: lo with its upper lanes replaced by hi's lower lanes; y: hi with its lower lanes replaced by lo's upper lanes
-        const u2s r = __builtin_amdgcn_permlane32_swap(lo[dw], hi[dw], false, false);
-        t0[dw] = r.x; t1[dw] = r.y;
-      }
-      o.a[par][0] = __builtin_bit_cast(h8, t0);
-      o.a[par][1] = __builtin_bit_cast(h8, t1);
-    }
+    for (int par = 0; par < 2; ++par) { o.a[par][0] = d.a[2 * par]; o.a[par][1] = d.a[2 * par + 1]; }
   };
 
   // activation scale of this lane's column of each 32-row block of the output (activation row 32 jb + lane % 32)
@@ -1742,15 +1736,16 @@ __global__ __launch_bounds__(GEMM_THREADS) void k_linear_gemm(const uint32_t* __
 #pragma unroll
   for (int jb = 0; jb < JB; ++jb) offs[jb] = 0.f;
   const float k1534 = cq == 0 ? 1534.f : 0.f;
-  // B operands: lane (activation row l32 of the 32-row block, k-group kg) reads 8 consecutive columns 16 tc + 8 kg .. + 7
-  const _Float16* b_lane = x_tile + l32 * GEMM_LD + 32 * cq + 8 * kg;
+  // B operands: lane (activation row l32 of the 32-row block, k-group kg) reads columns 0..7 (then 8..15) of tile column
+  // 2 cq + kg of the block
+  const _Float16* b_lane = x_tile + l32 * GEMM_LD + 32 * cq + 16 * kg;
 
   // products of one decoded step with the staged block in buffer xb
   auto multiply = [&](const Operands& o, int xb) {
     const _Float16* bp = b_lane + xb * GEMM_TILE_HALVES;
 #pragma unroll
     for (int jb = 0; jb < JB; ++jb) {
-      const h8 b0 = *(const h8*)(bp + jb * 32 * GEMM_LD), b1 = *(const h8*)(bp + jb * 32 * GEMM_LD + 16);
+      const h8 b0 = *(const h8*)(bp + jb * 32 * GEMM_LD), b1 = *(const h8*)(bp + jb * 32 * GEMM_LD + 8);
       acc[jb][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(o.a[0][0], b0, acc[jb][0], 0, 0, 0);
       acc[jb][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(o.a[1][0], b0, acc[jb][1], 0, 0, 0);
       acc[jb][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(o.a[0][1], b1, acc[jb][0], 0, 0, 0);
@@ -1764,6 +1759,10 @@ __global__ __launch_bounds__(GEMM_THREADS) void k_linear_gemm(const uint32_t* __
     decode_step<K>(sr, hist, d);
     prefetch(sr);
     form(d, cur);
+    // the operands exist HERE, in the half in which this wave decodes: without the pin the compiler sinks the whole
+    // decode (it touches no memory) across the barrier to its first use, into the half in which the wave multiplies
+#pragma unroll
+    for (int par = 0; par < 2; ++par) { asm volatile("" : "+v"(cur.a[par][0])); asm volatile("" : "+v"(cur.a[par][1])); }
   };
 
   // ---- A step is two halves with a barrier behind each.  The two waves that share a SIMD work in opposite halves: waves
@@ -1786,12 +1785,18 @@ __global__ __launch_bounds__(GEMM_THREADS) void k_linear_gemm(const uint32_t* __
       // every wave moves its pieces of block v + 1 to their buffer, and requests those of block v + 2, at the start of
       // the half in which it multiplies: the matrix instructions queue up behind and hide it
       const int xn = xb == GEMM_XBUFS - 1 ? 0 : xb + 1;
+      // (scheduling fences on both sides of the barriers: the decode touches no memory, so the compiler is otherwise
+      // free to move it across a barrier into the half in which the same wave multiplies)
       if constexpr (!LAG) { stage_store(xn, set); stage_load(c_begin + vstep + 3, set); multiply(cur, xb); } else decode_next(mine);
+      HTR_PIN();
       __syncthreads();
+      HTR_PIN();
       if constexpr (LAG) { stage_store(xn, set); stage_load(c_begin + vstep + 3, set); multiply(cur, xb); } else { if (more) decode_next(ahead); }
       xb = xn;
       ++vstep;
+      HTR_PIN();
       __syncthreads();
+      HTR_PIN();
     };
     int v = 0;
     for (; v + P < nsteps; v += P) {

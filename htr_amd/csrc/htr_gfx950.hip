@@ -1765,12 +1765,14 @@ __global__ __launch_bounds__(GEMM_THREADS) void k_linear_gemm(const uint32_t* __
     for (int par = 0; par < 2; ++par) { asm volatile("" : "+v"(cur.a[par][0])); asm volatile("" : "+v"(cur.a[par][1])); }
   };
 
-  // ---- A step is two halves with a barrier behind each.  The two waves that share a SIMD work in opposite halves: waves
-  // 0..3 multiply block v in the first half and decode block v + 1 in the second, waves 4..7 decode block v in the
-  // first half and multiply it in the second.  So in every half each SIMD has one wave on the matrix unit and one on
-  // the vector unit, and the two run side by side (matrix instructions of one wave do not hold up the vector
-  // instructions of another).  Block v's activations are in buffer v % 3, stored during step v - 1; block v + 1's go
-  // from registers to their buffer during step v, when block v + 2 is requested.
+  // ---- A step has two halves and ONE barrier, at its end.  The two waves that share a SIMD work in opposite order:
+  // waves 0..3 multiply block v in the first half and decode block v + 1 in the second, waves 4..7 decode block v
+  // first and multiply it second.  So most of the time each SIMD has one wave on the matrix unit and one on the vector
+  // unit, and the two run side by side (matrix instructions of one wave do not hold up the vector instructions of
+  // another); between barriers the waves run freely, which costs nothing: the loop is as fast as with no barrier at all
+  // (a second barrier between the halves cost 7 %).  Block v's activations are in buffer v % 3, stored by every wave
+  // during step v - 1 (so complete at that step's barrier); block v + 1's go from registers to their buffer during
+  // step v, whose previous content (block v - 2) was last read two barriers ago; block v + 3 is requested then.
   // (Two copies of the loop, chosen once per wave: with the choice inside the loop the compiler keeps the registers of
   // both kinds of half alive side by side and spills.)
   static_assert(P == 2 || P == 4, "stream buffers rotate with the unrolled loop");
@@ -1785,11 +1787,8 @@ __global__ __launch_bounds__(GEMM_THREADS) void k_linear_gemm(const uint32_t* __
       // every wave moves its pieces of block v + 1 to their buffer, and requests those of block v + 2, at the start of
       // the half in which it multiplies: the matrix instructions queue up behind and hide it
       const int xn = xb == GEMM_XBUFS - 1 ? 0 : xb + 1;
-      // (scheduling fences on both sides of the barriers: the decode touches no memory, so the compiler is otherwise
-      // free to move it across a barrier into the half in which the same wave multiplies)
+      // (scheduling fences between the halves and around the barrier: the halves stay in the order written)
       if constexpr (!LAG) { stage_store(xn, set); stage_load(c_begin + vstep + 3, set); multiply(cur, xb); } else decode_next(mine);
-      HTR_PIN();
-      __syncthreads();
       HTR_PIN();
       if constexpr (LAG) { stage_store(xn, set); stage_load(c_begin + vstep + 3, set); multiply(cur, xb); } else { if (more) decode_next(ahead); }
       xb = xn;

@@ -23,23 +23,22 @@ GROUP_MAX_M = _native.MAX_GROUP_ROWS      # rows per entry of a grouped launch
 NSPLIT = int(os.environ.get("HTR_NSPLIT", "0"))
 # Above a number of activation rows the weight is dequantized once to the original basis (bf16) and a library GEMM does
 # the product, as the reference does for prefill (HTR_PREFILL="w", htr/ops.py:52-54,89-93); up to it, fused launches
-# run (the reference's HTR_GEMV_LOOP_MAX, htr/ops.py:59-61): up to 128 rows the batched decode kernel; beyond, either the
+# run (the reference's HTR_GEMV_LOOP_MAX, htr/ops.py:59-61): up to 128 rows the batched decode kernel; beyond, the
 # fused decode -> matrix-unit kernel in ONE launch (it re-decodes the weight once per 96 activation rows, so it pays while
-# few such tiles cover the input and the grid stays within the chip) or launches of 128 rows, whichever was faster.
+# few such tiles cover the input).
 # Measured on MI355X (K4, eager, us; one fused launch incl. its rotation launch / launches of 128 rows / dequantize + GEMM):
-#   14336x4096: 160 rows 47 / 63 / 77, 192 rows 50 / 73 / 81, 256 rows 87 / 81 / 90, 384 rows 98 / 129 / 97
-#   4096x14336: 160 rows 52 / 61 / 117, 192 rows 55 / 68 / 127, 256 rows 89 / 88 / 96, 384 rows 95 / 133 / 117, 512 rows 147 / 162 / 129
-#   6144x4096:  160 rows 35 / 46 / 48, 192 rows 37 / 50 / 51, 256 rows 45 / 58 / 59, 384 rows 49 / 83 / 53, 512 rows 87 / 109 / 56
-#   4096x4096:  160 rows 32 / 37 / 41, 192 rows 33 / 51 / 44, 256 rows 37 / 46 / 37, 384 rows 41 / 69 / 40, 512 rows 49 / 90 / 45
-# So: one fused launch while its tiles x the weight's row blocks fit the chip in one round, up to 384 rows (192 on a
-# matrix as small as 4096x4096, whose dequantization is cheap); two launches of 128 rows where a third tile would start
-# a second round (14336x4096 at 193..256 rows); else dequantize.  HTR_GEMV_LOOP_MAX overrides the row limit for every
-# shape (launches of LAUNCH_MAX_M rows up to it).
+#   14336x4096: 160 rows 43 / 62 / 76, 192 rows 45 / 70 / 80, 256 rows 79 / 82 / 89, 384 rows 92 / 129 / 95, 512 rows 136 / 159 / 99
+#   4096x14336: 160 rows 49 / 62 / 115, 192 rows 52 / 65 / 126, 256 rows 76 / 86 / 93, 384 rows 89 / 132 / 115, 512 rows 137 / 166 / 127
+#   6144x4096:  160 rows 34 / 45 / 47, 192 rows 36 / 50 / 51, 256 rows 42 / 57 / 59, 384 rows 46 / 83 / 53, 512 rows 78 / 112 / 56
+#   4096x4096:  160 rows 31 / 45 / 41, 192 rows 32 / 40 / 44, 256 rows 35 / 47 / 37, 384 rows 40 / 69 / 41, 512 rows 46 / 90 / 44
+# So: one fused launch up to 384 rows on matrices from 4096x4096 up, dequantize beyond (and from 129 rows on smaller
+# matrices, whose dequantization is cheap and which were not measured).  HTR_GEMV_LOOP_MAX overrides the row limit for
+# every shape (launches of LAUNCH_MAX_M rows up to it).
 _LOOP_MAX_ENV = os.environ.get("HTR_GEMV_LOOP_MAX")
 GEMV_LOOP_MAX = None if _LOOP_MAX_ENV is None else int(_LOOP_MAX_ENV)
 ONE_LAUNCH = _native.MAX_BATCH
-_TILE_ROWS = 96          # activation rows per tile of the fused GEMM kernel
-_CHIP_WORKGROUPS = 256   # one workgroup per compute unit of the MI355X the table above was measured on
+FUSED_GEMM_MAX_ROWS = 384
+FUSED_GEMM_MIN_WEIGHTS = 4096 * 4096
 
 
 def fused_rows_per_launch(m, n, M):
@@ -48,12 +47,8 @@ def fused_rows_per_launch(m, n, M):
         return LAUNCH_MAX_M if M <= GEMV_LOOP_MAX else 0
     if M <= _native.MAX_ROWS_PER_TILE:
         rows = _native.MAX_ROWS_PER_TILE
-    elif m * n < 6144 * 4096:
-        rows = ONE_LAUNCH if (m * n >= 4096 * 4096 and M <= 192) else 0
-    elif M <= 384 and (m // 128) * -(-M // _TILE_ROWS) <= _CHIP_WORKGROUPS:
-        rows = ONE_LAUNCH
     else:
-        rows = _native.MAX_ROWS_PER_TILE if M <= 256 else 0
+        rows = ONE_LAUNCH if (m * n >= FUSED_GEMM_MIN_WEIGHTS and M <= FUSED_GEMM_MAX_ROWS) else 0
     return min(rows, LAUNCH_MAX_M)
 
 
@@ -61,9 +56,7 @@ def fused_max_rows(m, n):
     """Activation rows up to which the fused kernels take an [m, n] linear; more rows go to dequantize + library GEMM."""
     if GEMV_LOOP_MAX is not None:
         return GEMV_LOOP_MAX
-    if m * n < 6144 * 4096:
-        return 192 if m * n >= 4096 * 4096 else _native.MAX_ROWS_PER_TILE
-    return 384 if (m // 128) * 4 <= _CHIP_WORKGROUPS else 256
+    return FUSED_GEMM_MAX_ROWS if m * n >= FUSED_GEMM_MIN_WEIGHTS else _native.MAX_ROWS_PER_TILE
 
 
 # How inputs beyond GEMV_LOOP_MAX rows are multiplied (the reference's HTR_PREFILL, htr/ops.py:52-54): "w" = dequantize

@@ -419,17 +419,14 @@ def test_more_than_128_rows_through_ops_with_bias(dev, oracle, dtype, monkeypatc
     assert _rel(y.float().cpu().numpy(), ref) <= tol
 
 
-def test_fused_row_limit_follows_the_shape(dev, oracle):
+def test_fused_row_limit_follows_the_shape(dev, oracle, monkeypatch):
     """ops.linear takes one launch of the fused GEMM kernel, launches of 128 rows or dequantize + GEMM depending on shape
     and row count; all three give the same product."""
     from htr_amd import ops
     big = ops.ONE_LAUNCH
-    assert ops.fused_max_rows(4096, 4096) == 192 and ops.fused_max_rows(14336, 4096) == 256 and ops.fused_max_rows(1024, 4096) == 128
-    assert ops.fused_max_rows(4096, 14336) == 384 and ops.fused_max_rows(6144, 4096) == 384
-    assert [ops.fused_rows_per_launch(14336, 4096, M) for M in (1, 128, 129, 192, 193, 256, 257)] == [128, 128, big, big, 128, 128, 0]
-    assert [ops.fused_rows_per_launch(4096, 14336, M) for M in (129, 384, 385)] == [big, big, 0]
-    assert [ops.fused_rows_per_launch(6144, 4096, M) for M in (129, 384, 385)] == [big, big, 0]
-    assert [ops.fused_rows_per_launch(4096, 4096, M) for M in (129, 192, 193)] == [big, big, 0]
+    assert ops.fused_max_rows(4096, 4096) == 384 and ops.fused_max_rows(14336, 4096) == 384 and ops.fused_max_rows(1024, 4096) == 128
+    assert [ops.fused_rows_per_launch(14336, 4096, M) for M in (1, 128, 129, 384, 385)] == [128, 128, big, big, 0]
+    assert [ops.fused_rows_per_launch(4096, 4096, M) for M in (129, 384, 385)] == [big, big, 0]
     assert ops.fused_rows_per_launch(2048, 2048, 129) == 0
     print("gemm kernel at the policy's shape", flush=True)
     qw, sc, su, sv, x = _case(14336, 4096, 4, 192, 9200)
@@ -437,10 +434,14 @@ def test_fused_row_limit_follows_the_shape(dev, oracle):
     ref = _ref(oracle, qw, sc, su, sv, x)
     y = ops.linear_f32out(x.to(dev), *d).cpu().numpy()                                # one launch of the GEMM kernel
     assert _rel(y, ref) <= REL_TOL
+    monkeypatch.setattr(ops, "GEMV_LOOP_MAX", 1 << 30)
+    monkeypatch.setattr(ops, "LAUNCH_MAX_M", 128)
     x200 = torch.cat([x, x[:8]])
     y2 = ops.linear_f32out(x200.to(dev), *d).cpu().numpy()                            # 128 + 72 rows, batched kernel
     assert _rel(y2[:192], ref) <= REL_TOL and _rel(y2[192:], ref[:8]) <= REL_TOL
-    y3 = ops.linear(torch.cat([x, x[:100]]).to(dev), *d).float().cpu().numpy()        # 292 rows: dequantize + GEMM
+    monkeypatch.setattr(ops, "GEMV_LOOP_MAX", None)
+    monkeypatch.setattr(ops, "LAUNCH_MAX_M", ops.ONE_LAUNCH)
+    y3 = ops.linear(torch.cat([x, x, x[:100]]).to(dev), *d).float().cpu().numpy()     # 484 rows: dequantize + GEMM
     assert _rel(y3[:192], ref) <= 2.0 ** -6
 
 

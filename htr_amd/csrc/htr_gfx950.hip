@@ -605,7 +605,7 @@ constexpr int FLAG_LANE_LEN_SHIFT = 8; // with FLAG_LANES: grid / 8 in the bits 
 
 // ANCHOR = 1 is the same kernel with the decode compiled out (stream, rotation, products, hand-over and output side stay;
 // the results are meaningless): a timing anchor that tells how much of a launch is the decode.
-template <int K, int MB, int P, int D, bool PREROT, int RP, int ANCHOR = 0>
+template <int K, int MB, int P, int D, bool PREROT, int RP, int ANCHOR = 0, bool PACE = false>
 __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restrict__ qw_a, const void* __restrict__ x_a,
                                                        const uint8_t* __restrict__ su_a, float* __restrict__ part_a,
                                                        int m, int n, int M_a, int chunk, int flags,
@@ -1015,7 +1015,20 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
     if (i < nsteps) consume(pre[i], true);
   DecodedStep<K> cur = pre[D - 1];
   int v = D - 1;
+  // The two waves that share a SIMD (w and w + 4) compete for its issue slots, and between equals the arbiter favours the
+  // older one: left alone, waves 0..3 run ahead, leave the loop when the others have 40 % of their steps to go, and
+  // those finish at the rate of one wave per SIMD (an instruction every five cycles instead of two waves' three).  In
+  // the PACE instantiation the younger waves take the higher priority for two groups of P steps out of every four:
+  // both keep pace, and the SIMD has two waves to issue from until the end (gate_up 28672x4096: 19.1 -> 17.7 us).  It
+  // is a variant of its own, chosen by the launcher for long chunks, because it does not pay everywhere (short chunks,
+  // many rows with many contributors per row block) and its mere presence in the code changed how the compiler laid
+  // out the short-chunk kernels.
   for (; v + P < nsteps; v += P) {
+    if constexpr (PACE) {
+      if (w >= 4) {
+        if ((v / P) & 2) __builtin_amdgcn_s_setprio(0); else __builtin_amdgcn_s_setprio(1);
+      }
+    }
 #pragma unroll
     for (int pp = 0; pp < P; ++pp) {
       StreamRegs<K>& nxt = buf[(pp + D) % P];
@@ -1024,6 +1037,7 @@ __global__ __launch_bounds__(WG_THREADS) void k_linear(const uint32_t* __restric
       prefetch(nxt);
     }
   }
+  if constexpr (PACE) __builtin_amdgcn_s_setprio(0);
 #pragma unroll
   for (int pp = 0; pp < P; ++pp) {
     if (v + pp < nsteps) {
@@ -2558,14 +2572,25 @@ struct LinearLaunch {
   LinearTail tail;
 };
 
-template <int K, int MB, bool DEEP, bool PREROT, int RP = 1> int launch_linear_v(const LinearLaunch& a, int grid, size_t lds, hipStream_t st) {
+template <int K, int MB, bool DEEP, bool PREROT, int RP = 1, bool PACE = false>
+int launch_linear_v(const LinearLaunch& a, int grid, size_t lds, hipStream_t st) {
   constexpr int P = K <= 4 ? 4 : (K <= 6 ? 3 : 2);          // wave-steps of weights in flight
   constexpr int D = DEEP && P >= 4 ? 4 : 2;                 // steps decoded ahead of the activation exchange
   lds = balanced_lds_request(lds, grid * a.problems);
-  HTR_CHECK_HIP((allow_full_lds<k_linear<K, MB, P, D, PREROT, RP>>()));
-  HTR_CHECK_HIP(launch_kernel(k_linear<K, MB, P, D, PREROT, RP>, dim3(grid, a.problems), dim3(WG_THREADS), lds, st, a.qw, a.x, a.su, a.part,
-                              a.m, a.n, a.M, a.chunk, a.flags, a.nblk_magic, a.tail));
+  HTR_CHECK_HIP((allow_full_lds<k_linear<K, MB, P, D, PREROT, RP, 0, PACE>>()));
+  HTR_CHECK_HIP(launch_kernel(k_linear<K, MB, P, D, PREROT, RP, 0, PACE>, dim3(grid, a.problems), dim3(WG_THREADS), lds, st, a.qw, a.x, a.su,
+                              a.part, a.m, a.n, a.M, a.chunk, a.flags, a.nblk_magic, a.tail));
   return HTR_OK;
+}
+// Where the two waves of a SIMD are kept in step by alternating priorities (k_linear's PACE): chunks of twelve steps and
+// more, one launch (not a group), and either up to four activation rows or at most two chunks per row block.
+// Measured on MI355X, K4, us without -> with: 28672x4096 1 row 19.1 -> 17.7, 4 rows 22.0 -> 20.5, 8 rows 23.3 -> 23.5;
+// 14336x4096 1 / 4 / 8 rows 12.3 -> 11.8, 13.7 -> 12.9, 15.8 -> 14.4; 4096x14336 (eight chunks per row block) 1 / 4 / 6 /
+// 8 rows 11.9 -> 11.2, 12.9 -> 12.7, 14.0 -> 14.1, 14.9 -> 16.0; 6144x4096 8 rows (chunks of 8) 10.0 -> 13.8.
+inline bool paced(const LinearLaunch& a) {
+  static const bool on = getenv("HTR_PACE") == nullptr || atoi(getenv("HTR_PACE")) != 0;
+  const int nblk = a.n / 128;
+  return on && a.problems == 1 && a.chunk >= 12 && (a.M <= 4 || (nblk + a.chunk - 1) / a.chunk <= 2);
 }
 // Short chunks are decoded completely ahead of the activation exchange (more registers, so only for one activation
 // block and chunks whose prologue latency is a large part of the kernel); long chunks prefer occupancy.
@@ -2573,7 +2598,10 @@ template <int K, bool PREROT> int launch_linear_kr(const LinearLaunch& a, int mb
   const bool deep = a.chunk <= 8;
   if constexpr (!PREROT) {                 // more pairs than one pass rotates: the variant with several passes (up to 8 rows)
     const int nblk = a.n / 128;
-    if (mb == 1 && a.M * (a.chunk < nblk ? a.chunk : nblk) > ROT_PAIRS) return launch_linear_v<K, 1, false, false, MAX_ROT_PASSES>(a, grid, lds, st);
+    if (mb == 1 && a.M * (a.chunk < nblk ? a.chunk : nblk) > ROT_PAIRS)
+      return paced(a) ? launch_linear_v<K, 1, false, false, MAX_ROT_PASSES, true>(a, grid, lds, st)
+                      : launch_linear_v<K, 1, false, false, MAX_ROT_PASSES>(a, grid, lds, st);
+    if (mb == 1 && !deep && paced(a)) return launch_linear_v<K, 1, false, false, 1, true>(a, grid, lds, st);
   }
   switch (mb) {
     case 1: return deep ? launch_linear_v<K, 1, true, PREROT>(a, grid, lds, st) : launch_linear_v<K, 1, false, PREROT>(a, grid, lds, st);

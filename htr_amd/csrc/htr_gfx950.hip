@@ -1641,18 +1641,21 @@ __global__ __launch_bounds__(WG_THREADS, MG <= 2 && !ROT ? 4 : 2) void k_linear_
 // is undone; with S > 1 the last split of a row block collects the others' tiles and finishes: row scale, output H128,
 // sign, bias, cast.
 constexpr int GEMM_THREADS = WG_THREADS;
-constexpr int GEMM_JB = 3;                                     // 32-row blocks of activation rows per tile
-constexpr int GEMM_ROWS = 32 * GEMM_JB;                        // activation rows per tile
+// activation rows per tile = 32 JB, JB = 3 or 4: with 96 rows the weight is decoded once more per 96 rows but a step is
+// shorter and the activations travel two steps ahead in two register sets; 128 rows need the registers (one set, one
+// step ahead, two stream buffers) and pay where they save a round of workgroups.  The planner chooses.
 constexpr int GEMM_LD = 128 + 8;                               // halves per row of a staged activation block: 16-byte rows, 4 banks of shift
-constexpr int GEMM_TILE_HALVES = GEMM_ROWS * GEMM_LD;
 constexpr int GEMM_XBUFS = 3;
 constexpr int GEMM_FIN_LD = 128 + 4;                           // floats per activation row of the output in LDS
-constexpr size_t GEMM_FIN_BYTES = (size_t)2 * GEMM_ROWS * GEMM_FIN_LD * 4;            // two copies of the output (column quarters 0, 2 | 1, 3)
-constexpr size_t GEMM_X_BYTES = (size_t)GEMM_XBUFS * GEMM_TILE_HALVES * 2 + GEMM_XBUFS * GEMM_ROWS * 4;
-constexpr size_t GEMM_LDS_BYTES = (GEMM_FIN_BYTES > GEMM_X_BYTES ? GEMM_FIN_BYTES : GEMM_X_BYTES) + 16;
+constexpr size_t gemm_lds_bytes(int jb) {
+  const size_t rows = (size_t)32 * jb;
+  const size_t fin = 2 * rows * GEMM_FIN_LD * 4;               // two copies of the output (column quarters 0, 2 | 1, 3)
+  const size_t xb = GEMM_XBUFS * rows * GEMM_LD * 2 + GEMM_XBUFS * rows * 4;
+  return (fin > xb ? fin : xb) + 16;
+}
 typedef float f16v __attribute__((ext_vector_type(16)));
 
-template <int K, int P>
+template <int K, int P, int JB>
 __global__ __launch_bounds__(GEMM_THREADS) void k_linear_gemm(const uint32_t* __restrict__ qw, float* __restrict__ part,
                                                                  int m, int n, int M, int S, int flags, const LinearTail t) {
   extern __shared__ __align__(16) unsigned char lds[];
@@ -1661,6 +1664,9 @@ __global__ __launch_bounds__(GEMM_THREADS) void k_linear_gemm(const uint32_t* __
   const int rh = w & 1, cq = w >> 1;
   const int nblk = n >> 7;
   const int s_idx = blockIdx.x, rb = blockIdx.y, mt = blockIdx.z;
+  constexpr int GEMM_ROWS = 32 * JB, GEMM_TILE_HALVES = GEMM_ROWS * GEMM_LD;
+  constexpr size_t GEMM_LDS_BYTES = gemm_lds_bytes(JB);
+  constexpr int XSETS = JB <= 3 ? 2 : 1;                         // register sets of activations in flight = steps ahead
   const int j0 = mt * GEMM_ROWS, rows = min(GEMM_ROWS, M - j0);  // this tile's activation rows
   const int cb = (nblk + S - 1) / S;
   const int c_begin = s_idx * cb, c_end = min(nblk, c_begin + cb);
@@ -1689,8 +1695,8 @@ __global__ __launch_bounds__(GEMM_THREADS) void k_linear_gemm(const uint32_t* __
     piece_lds[i] = prow * GEMM_LD + pg * 8;
   }
   const int sum_src = tid < rows ? ((j0 + tid) * nblk) * 16 : -1;          // {even tiles, odd tiles, ...} of block 0
-  u4 xg[2][NPT];
-  u2 xsg[2];
+  u4 xg[XSETS][NPT];
+  u2 xsg[XSETS];
   auto stage_load = [&](int blk, int set) {    // block index in the row; beyond the split: zeros, no traffic
     HTR_PIN();
     const bool live = blk < c_end;
@@ -1706,7 +1712,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void k_linear_gemm(const uint32_t* __
     if (tid < GEMM_ROWS) s_xs[xb * GEMM_ROWS + tid] = __uint_as_float(xsg[set].x) + __uint_as_float(xsg[set].y);
   };
   stage_load(c_begin, 0);
-  stage_load(c_begin + 1, 1);
+  if constexpr (XSETS == 2) stage_load(c_begin + 1, 1);
 
   // ---- the weight stream: lane = (tile column 2 cq + lane / 32, strip 4 rh + lane % 32 / 8, row pair q = lane % 8); the 8
   // lanes of a tile are consecutive, so the history exchange is the one of k_linear.  One descriptor over the row block's
@@ -1744,7 +1750,6 @@ __global__ __launch_bounds__(GEMM_THREADS) void k_linear_gemm(const uint32_t* __
   };
 
   // activation scale of this lane's column of each 32-row block of the output (activation row 32 jb + lane % 32)
-  constexpr int JB = GEMM_ROWS / 32;
   f16v acc[JB][2];
 #pragma unroll
   for (int jb = 0; jb < JB; ++jb)
@@ -1799,8 +1804,8 @@ __global__ __launch_bounds__(GEMM_THREADS) void k_linear_gemm(const uint32_t* __
   auto run = [&](auto lag_c) {
     constexpr bool LAG = decltype(lag_c)::value;
     if constexpr (!LAG) decode_next(buf[0]);
-    stage_store(0, 0);                                           // block 0 (set 0) to buffer 0; block 2 requested into set 0
-    stage_load(c_begin + 2, 0);
+    stage_store(0, 0);                                           // block 0 (set 0) to buffer 0; the next block not yet requested into set 0
+    stage_load(c_begin + XSETS, 0);
     __syncthreads();
     int xb = 0, vstep = 0;                                       // buffer of the step being multiplied, its index
     auto step = [&](StreamRegs<K>& mine, StreamRegs<K>& ahead, bool more, int set) {      // set: register set of block v + 1
@@ -1808,9 +1813,9 @@ __global__ __launch_bounds__(GEMM_THREADS) void k_linear_gemm(const uint32_t* __
       // the half in which it multiplies: the matrix instructions queue up behind and hide it
       const int xn = xb == GEMM_XBUFS - 1 ? 0 : xb + 1;
       // (scheduling fences between the halves and around the barrier: the halves stay in the order written)
-      if constexpr (!LAG) { stage_store(xn, set); stage_load(c_begin + vstep + 3, set); multiply(cur, xb); } else decode_next(mine);
+      if constexpr (!LAG) { stage_store(xn, set % XSETS); stage_load(c_begin + vstep + 1 + XSETS, set % XSETS); multiply(cur, xb); } else decode_next(mine);
       HTR_PIN();
-      if constexpr (LAG) { stage_store(xn, set); stage_load(c_begin + vstep + 3, set); multiply(cur, xb); } else { if (more) decode_next(ahead); }
+      if constexpr (LAG) { stage_store(xn, set % XSETS); stage_load(c_begin + vstep + 1 + XSETS, set % XSETS); multiply(cur, xb); } else { if (more) decode_next(ahead); }
       xb = xn;
       ++vstep;
       HTR_PIN();
@@ -2669,17 +2674,18 @@ inline bool make_batch_plan(int m, int n, int M, int want_S, BatchPlan& bp) {
 
 // ---- GEMM kernel (more than 128 rows): tiles of GEMM_ROWS activation rows in the grid's z, split S of the column blocks
 // while the grid stays within one workgroup per compute unit (256 registers per lane leave room for one)
-struct GemmPlan { int S, cb, mtiles, wgs; };
+struct GemmPlan { int S, cb, mtiles, wgs, jb; };
 constexpr int GEMM_MIN_M = HTR_MAX_ROWS_PER_TILE + 1;       // rows from which the library policy takes the GEMM kernel
-inline bool make_gemm_plan(int m, int n, int M, int want_S, GemmPlan& gp) {
-  const int nblk = n / 128, rbs = m / 128;
+inline bool gemm_plan_for(int m, int n, int M, int want_S, int jb, GemmPlan& gp) {
+  const int nblk = n / 128, rbs = m / 128, rows = 32 * jb;
   if ((long)M * n * 2 >= (1L << 31)) return false;          // the kernel addresses the rotated activations with 32-bit byte offsets
-  gp.mtiles = (M + GEMM_ROWS - 1) / GEMM_ROWS;
+  gp.jb = jb;
+  gp.mtiles = (M + rows - 1) / rows;
   if (gp.mtiles > 65535) return false;
   const long base = (long)rbs * gp.mtiles;
   const int cus = num_cu();
   const int by_cus = cus / base > 1 ? (int)(cus / base) : 1;
-  const int limit = want_S > 0 ? want_S : (by_cus < 8 ? by_cus : 8);
+  const int limit = want_S > 0 ? want_S : (by_cus < 4 ? by_cus : 4);
   bool found = false;
   for (int S = 1; S <= nblk && S <= limit && S <= 8; ++S) {
     const int cb = (nblk + S - 1) / S;
@@ -2689,11 +2695,32 @@ inline bool make_gemm_plan(int m, int n, int M, int want_S, GemmPlan& gp) {
   }
   return found;
 }
+// Tile height by a cost model in microseconds fitted to MI355X (K4): rounds of workgroups over the CUs x (steps per
+// workgroup x 0.94 us with 96-row tiles, 1.16 us with 128-row tiles, + 10 us of fixed cost, + 4 + 1.5 (S - 1) us for the
+// exchange between S column splits).  128-row tiles win where they save a round (14336x4096 at 256 rows: two tiles
+// fill the chip once, 49 us, where three tiles of 96 rows take 73) or allow more splits of long rows (4096x14336 at 256
+// rows: 55 against 64); 96-row tiles win otherwise (14336x4096 at 192 rows: 40 against 47; at 384 rows: 79 against 94).
+// want_jb: 0 = this policy, 3 or 4 = that tile height.  By policy at most four splits (eight cost more than they save).
+inline double gemm_plan_cost(const GemmPlan& gp) {
+  const int cus = num_cu();
+  const int rounds = (gp.wgs + cus - 1) / cus;
+  return rounds * (gp.cb * (gp.jb == 3 ? 0.94 : 1.16) + 10.0 + (gp.S > 1 ? 4.0 + 1.5 * (gp.S - 1) : 0.0));
+}
+inline bool make_gemm_plan(int m, int n, int M, int want_S, int want_jb, GemmPlan& gp) {
+  if (want_jb == 3 || want_jb == 4) return gemm_plan_for(m, n, M, want_S, want_jb, gp);
+  GemmPlan a, b;
+  const bool oka = gemm_plan_for(m, n, M, want_S, 3, a), okb = gemm_plan_for(m, n, M, want_S, 4, b);
+  if (!oka && !okb) return false;
+  gp = oka && (!okb || gemm_plan_cost(a) <= gemm_plan_cost(b)) ? a : b;
+  return true;
+}
 // workspace of the GEMM kernel: one flag word per workgroup in the zeroed half; rotated activations and the exchange tiles
 // (only with column splits) in the scratch half
 inline size_t gemm_scratch_bytes(int n, int M, const GemmPlan& gp) {
-  return prerot_bytes(n, M) + (gp.S > 1 ? (size_t)gp.wgs * GEMM_ROWS * 128 * sizeof(float) : 0);
+  return prerot_bytes(n, M) + (gp.S > 1 ? (size_t)gp.wgs * (32 * gp.jb) * 128 * sizeof(float) : 0);
 }
+// nsplit bits 20 and 21 with the GEMM kernel: tiles of 96 or of 128 activation rows (neither: the policy above)
+inline int gemm_want_jb(int nsplit) { return nsplit > 0 ? ((nsplit >> 20) & 1 ? 3 : ((nsplit >> 21) & 1 ? 4 : 0)) : 0; }
 // nsplit bit 28: the GEMM kernel with the split in the low bits (0 = its own policy); otherwise from GEMM_MIN_M rows
 inline bool wants_gemm(int M, int nsplit) { return nsplit > 0 ? (nsplit & (1 << 28)) != 0 : M >= GEMM_MIN_M; }
 
@@ -2785,7 +2812,7 @@ size_t htr_workspace_bytes(int m, int n, int K, int M, int nsplit) {
   if (K < 2 || K > 8 || !shape_ok(m, n) || M < 1 || M > HTR_MAX_BATCH) return 0;
   if (wants_gemm(M, nsplit)) {
     GemmPlan gp;
-    if (!make_gemm_plan(m, n, M, nsplit > 0 ? nsplit & 0xFFFFF : 0, gp)) return 0;
+    if (!make_gemm_plan(m, n, M, nsplit > 0 ? nsplit & 0xFFFFF : 0, gemm_want_jb(nsplit), gp)) return 0;
     return ws_need((size_t)gp.wgs * sizeof(uint32_t), gemm_scratch_bytes(n, M, gp));
   }
   if (M > HTR_MAX_ROWS_PER_TILE) return 0;       // the other kernels take up to 128 rows
@@ -2807,8 +2834,8 @@ int htr_linear_plan(int m, int n, int K, int M, int nsplit, int* out6) {
   if (M < 1 || M > HTR_MAX_BATCH) return HTR_ERR_BATCH;
   if (wants_gemm(M, nsplit)) {
     GemmPlan gp;
-    if (!make_gemm_plan(m, n, M, nsplit > 0 ? nsplit & 0xFFFFF : 0, gp)) return HTR_ERR_SPLIT;
-    out6[0] = gp.cb; out6[1] = gp.wgs; out6[2] = gp.mtiles; out6[3] = gp.S; out6[4] = 1; out6[5] = (int)GEMM_LDS_BYTES;
+    if (!make_gemm_plan(m, n, M, nsplit > 0 ? nsplit & 0xFFFFF : 0, gemm_want_jb(nsplit), gp)) return HTR_ERR_SPLIT;
+    out6[0] = gp.cb; out6[1] = gp.wgs; out6[2] = gp.mtiles; out6[3] = gp.S; out6[4] = 1; out6[5] = (int)gemm_lds_bytes(gp.jb);
     return HTR_OK;
   }
   if (M > HTR_MAX_ROWS_PER_TILE) return HTR_ERR_BATCH;
@@ -2866,7 +2893,7 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
     return HTR_ERR_ALIGN;
   if (wants_gemm(M, nsplit)) {
     GemmPlan gp;
-    if (!make_gemm_plan(m, n, M, nsplit > 0 ? nsplit & 0xFFFFF : 0, gp)) return HTR_ERR_SPLIT;
+    if (!make_gemm_plan(m, n, M, nsplit > 0 ? nsplit & 0xFFFFF : 0, gemm_want_jb(nsplit), gp)) return HTR_ERR_SPLIT;
     const size_t need = htr_workspace_bytes(m, n, K, M, nsplit);
     if (!workspace || workspace_bytes < need || ((uintptr_t)workspace & 255)) return HTR_ERR_WORKSPACE;
     unsigned char* wsp = (unsigned char*)workspace + ws_half(workspace_bytes);
@@ -2888,9 +2915,15 @@ int htr_linear(const void* qweight, const void* scales, const void* su, const vo
     const int flg = x_dtype | (y_dtype << 2);
 #define HTR_LAUNCH_GEMM(KK_, PP_)                                                                                          \
     {                                                                                                                      \
-      HTR_CHECK_HIP((allow_full_lds<k_linear_gemm<KK_, PP_>>()));                                                          \
-      HTR_CHECK_HIP(launch_kernel(k_linear_gemm<KK_, PP_>, dim3(gp.S, m / 128, gp.mtiles), dim3(GEMM_THREADS), GEMM_LDS_BYTES, st, \
-                                  qwp, flags, m, n, M, gp.S, flg, t));                                                     \
+      if (gp.jb == 3) {                                                                                                    \
+        HTR_CHECK_HIP((allow_full_lds<k_linear_gemm<KK_, PP_, 3>>()));                                                     \
+        HTR_CHECK_HIP(launch_kernel(k_linear_gemm<KK_, PP_, 3>, dim3(gp.S, m / 128, gp.mtiles), dim3(GEMM_THREADS),        \
+                                    gemm_lds_bytes(3), st, qwp, flags, m, n, M, gp.S, flg, t));                            \
+      } else {                                                                                                             \
+        HTR_CHECK_HIP((allow_full_lds<k_linear_gemm<KK_, 2, 4>>()));                                                       \
+        HTR_CHECK_HIP(launch_kernel(k_linear_gemm<KK_, 2, 4>, dim3(gp.S, m / 128, gp.mtiles), dim3(GEMM_THREADS),          \
+                                    gemm_lds_bytes(4), st, qwp, flags, m, n, M, gp.S, flg, t));                            \
+      }                                                                                                                    \
     }
     switch (K) {
       case 2: HTR_LAUNCH_GEMM(2, 4); break;

@@ -27,13 +27,13 @@ NSPLIT = int(os.environ.get("HTR_NSPLIT", "0"))
 # fused decode -> matrix-unit kernel in ONE launch (it re-decodes the weight once per 96 activation rows, so it pays while
 # few such tiles cover the input).
 # Measured on MI355X (K4, eager, us; one fused launch incl. its rotation launch / launches of 128 rows / dequantize + GEMM):
-#   14336x4096: 160 rows 43 / 62 / 76, 192 rows 45 / 70 / 80, 256 rows 79 / 82 / 89, 384 rows 92 / 129 / 95, 512 rows 136 / 159 / 99
-#   4096x14336: 160 rows 49 / 62 / 115, 192 rows 52 / 65 / 126, 256 rows 76 / 86 / 93, 384 rows 89 / 132 / 115, 512 rows 137 / 166 / 127
-#   6144x4096:  160 rows 34 / 45 / 47, 192 rows 36 / 50 / 51, 256 rows 42 / 57 / 59, 384 rows 46 / 83 / 53, 512 rows 78 / 112 / 56
-#   4096x4096:  160 rows 31 / 45 / 41, 192 rows 32 / 40 / 44, 256 rows 35 / 47 / 37, 384 rows 40 / 69 / 41, 512 rows 46 / 90 / 44
-# So: one fused launch up to 384 rows on matrices from 4096x4096 up, dequantize beyond (and from 129 rows on smaller
-# matrices, whose dequantization is cheap and which were not measured).  HTR_GEMV_LOOP_MAX overrides the row limit for
-# every shape (launches of LAUNCH_MAX_M rows up to it).
+#   14336x4096: 160 rows 44 / 64 / 77, 192 rows 45 / 68 / 81, 256 rows 55 / 81 / 89, 384 rows 93 / 126 / 95, 512 rows 119 / 167 / 102
+#   4096x14336: 160 rows 49 / 60 / 116, 192 rows 52 / 68 / 127, 256 rows 74 / 96 / 95, 384 rows 90 / 139 / 113, 512 rows 113 / 175 / 130
+#   6144x4096:  160 rows 34 / 43 / 48, 192 rows 35 / 49 / 51, 256 rows 42 / 57 / 59, 384 rows 46 / 88 / 54, 512 rows 56 / 113 / 56
+#   4096x4096:  160 rows 31 / 37 / 41, 192 rows 32 / 39 / 44, 256 rows 37 / 47 / 36, 384 rows 41 / 74 / 40, 512 rows 48 / 93 / 44
+# So: one fused launch up to 384 rows on matrices from 4096x4096 up (512 rows where the rows are long, n >= 8192),
+# dequantize beyond (and from 129 rows on smaller matrices, whose dequantization is cheap and which were not measured).
+# HTR_GEMV_LOOP_MAX overrides the row limit for every shape (launches of LAUNCH_MAX_M rows up to it).
 _LOOP_MAX_ENV = os.environ.get("HTR_GEMV_LOOP_MAX")
 GEMV_LOOP_MAX = None if _LOOP_MAX_ENV is None else int(_LOOP_MAX_ENV)
 ONE_LAUNCH = _native.MAX_BATCH
@@ -48,7 +48,7 @@ def fused_rows_per_launch(m, n, M):
     if M <= _native.MAX_ROWS_PER_TILE:
         rows = _native.MAX_ROWS_PER_TILE
     else:
-        rows = ONE_LAUNCH if (m * n >= FUSED_GEMM_MIN_WEIGHTS and M <= FUSED_GEMM_MAX_ROWS) else 0
+        rows = ONE_LAUNCH if (m * n >= FUSED_GEMM_MIN_WEIGHTS and M <= fused_max_rows(m, n)) else 0
     return min(rows, LAUNCH_MAX_M)
 
 
@@ -56,7 +56,9 @@ def fused_max_rows(m, n):
     """Activation rows up to which the fused kernels take an [m, n] linear; more rows go to dequantize + library GEMM."""
     if GEMV_LOOP_MAX is not None:
         return GEMV_LOOP_MAX
-    return FUSED_GEMM_MAX_ROWS if m * n >= FUSED_GEMM_MIN_WEIGHTS else _native.MAX_ROWS_PER_TILE
+    if m * n < FUSED_GEMM_MIN_WEIGHTS:
+        return _native.MAX_ROWS_PER_TILE
+    return 512 if n >= 8192 else FUSED_GEMM_MAX_ROWS
 
 
 # How inputs beyond GEMV_LOOP_MAX rows are multiplied (the reference's HTR_PREFILL, htr/ops.py:52-54): "w" = dequantize

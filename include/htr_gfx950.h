@@ -44,7 +44,7 @@ typedef enum {
 enum { HTR_BF16 = 0, HTR_F16 = 1, HTR_F32 = 2 };
 
 #define HTR_MAX_BATCH 2048      /* activation rows one htr_linear launch accepts */
-#define HTR_MAX_ROWS_PER_TILE 128   /* up to here one workgroup holds all rows; beyond, the GEMM kernel works in tiles of 96 rows */
+#define HTR_MAX_ROWS_PER_TILE 128   /* up to here one workgroup holds all rows; beyond, the GEMM kernel works in tiles of 96 or 128 rows */
 #define HTR_MAX_GROUP_ROWS 32   /* rows per problem of htr_linear_grouped (and of an explicit chunked plan, see nsplit) */
 #define HTR_MAX_GROUP 4096 /* problems one htr_linear_grouped launch accepts */
 
@@ -111,17 +111,19 @@ unsigned long long htr_stream_capture_id(void* stream);
  * over at most 8), dynamic LDS bytes}.  Entries 4 and 5 assume bf16 / f16 activations on a 16-byte boundary; float32 or
  * otherwise aligned activations always take the rotation launch and the staged kernel's LDS layout.
  * With more than HTR_MAX_ROWS_PER_TILE rows the fused decode -> matrix-unit (GEMM) kernel runs: the activations are
- * always rotated by a launch of their own, a workgroup owns one 128-row block of the weight, one tile of 96 activation
- * rows and one of S column splits, and the last split of a (row block, tile) adds up the others' partial tiles, which
- * travel through the workspace.  out6 = {column blocks per split, workgroups (= S x row blocks x row tiles), row tiles,
- * S, 1, dynamic LDS bytes}.  The reference has no such kernel: it dequantizes the weight and calls a library GEMM from
+ * always rotated by a launch of their own, a workgroup owns one 128-row block of the weight, one tile of 96 or of 128
+ * activation rows (the planner takes the height that saves a round of workgroups or allows more splits) and one of S
+ * column splits, and the last split of a (row block, tile) adds up the others' partial tiles, which travel through
+ * the workspace.  out6 = {column blocks per split, workgroups (= S x row blocks x row tiles), row tiles, S, 1, dynamic
+ * LDS bytes}.  The reference has no such kernel: it dequantizes the weight and calls a library GEMM from
  * these row counts on (htr/ops.py:89-93), which stays the better choice from a few hundred rows.
  * Plans are made for the current device's compute-unit count and LDS size (an unpartitioned MI355X where no device can
  * be asked); see htr_plan_device_override.
  * nsplit: 0 = library policy; otherwise the steps per workgroup of the chunked kernel (1 .. HTR_MAX_GROUP_ROWS rows;
  * bit 30 set: force the separate rotation launch), or, with bit 29 set, the batched kernel with that many column
  * splits in the low bits (0 = its own policy; up to HTR_MAX_ROWS_PER_TILE rows), or, with bit 28 set, the GEMM kernel
- * with that many column splits in the low bits (0 = its own policy, at most 8; any row count up to HTR_MAX_BATCH).
+ * with that many column splits in the low bits (0 = its own policy; at most 8; any row count up to HTR_MAX_BATCH) and
+ * tiles of 96 (bit 20) or 128 (bit 21) activation rows (neither: its own policy).
  */
 int htr_linear_plan(int m, int n, int K, int M, int nsplit, int* out6);
 

@@ -359,26 +359,30 @@ def test_small_batch_gemm_shapes(dev, oracle, K, M, m, n, monkeypatch):
 
 
 # ---- more than 128 activation rows in one launch: the fused decode -> matrix-unit kernel.  Row counts on both sides of
-# the 96-row tiles, every K, explicit column splits (nsplit = 2^28 + S) including the exchange between splits, bias and
-# all three output types, and a second call on the same workspace (the flags must be back at zero).
-_GEMM = [(4, 130, 256, 512, 0), (4, 200, 256, 512, 2), (4, 256, 384, 1024, 4), (4, 300, 256, 512, 1), (4, 257, 1024, 2048, 0),
-         (2, 129, 256, 384, 0), (3, 192, 384, 512, 2), (5, 193, 256, 512, 0), (6, 150, 256, 256, 1), (7, 288, 128, 384, 3),
-         (8, 161, 256, 512, 0), (4, 1000, 256, 256, 0), (4, 2048, 128, 256, 1), (4, 96, 256, 512, 1), (4, 40, 256, 384, 2)]
+# the tile edges, both tile heights (96 rows: nsplit bit 20, 128 rows: bit 21; neither: the planner's choice), every K,
+# explicit column splits (nsplit = 2^28 + S) including the exchange between splits, and a second call on the same
+# workspace (the flags must be back at zero).
+_GEMM = [(4, 130, 256, 512, 0, 0), (4, 200, 256, 512, 2, 3), (4, 256, 384, 1024, 4, 3), (4, 300, 256, 512, 1, 3), (4, 257, 1024, 2048, 0, 0),
+         (2, 129, 256, 384, 0, 3), (3, 192, 384, 512, 2, 3), (5, 193, 256, 512, 0, 0), (6, 150, 256, 256, 1, 3), (7, 288, 128, 384, 3, 3),
+         (8, 161, 256, 512, 0, 3), (4, 1000, 256, 256, 0, 0), (4, 2048, 128, 256, 1, 3), (4, 96, 256, 512, 1, 3), (4, 40, 256, 384, 2, 3),
+         (4, 200, 256, 512, 2, 4), (4, 256, 384, 1024, 4, 4), (4, 257, 256, 512, 1, 4), (2, 129, 256, 384, 0, 4), (3, 384, 384, 512, 2, 4),
+         (5, 385, 256, 512, 0, 4), (6, 150, 256, 256, 1, 4), (7, 288, 128, 384, 3, 4), (8, 128, 256, 512, 2, 4), (4, 2048, 128, 256, 1, 4)]
 
 
-@pytest.mark.parametrize("K,M,m,n,S", _GEMM)
-def test_more_than_128_rows_in_one_launch(dev, oracle, K, M, m, n, S):
+@pytest.mark.parametrize("K,M,m,n,S,T", _GEMM)
+def test_more_than_128_rows_in_one_launch(dev, oracle, K, M, m, n, S, T):
     import ctypes
     from htr_amd import _native
-    print(f"gemm kernel K={K} M={M} {m}x{n} S={S}", flush=True)
+    print(f"gemm kernel K={K} M={M} {m}x{n} S={S} tile={T}", flush=True)
     L = _native.lib()
-    nsplit = (1 << 28) | S if (S or M <= 128) else 0
+    nsplit = ((1 << 28) | S | {0: 0, 3: 1 << 20, 4: 1 << 21}[T]) if (S or T or M <= 128) else 0
     qw, sc, su, sv, x = _case(m, n, K, M, 9000 + 17 * K + M)
     d = [t.to(dev) for t in (qw, sc, su, sv)]
     xd = x.to(dev)
     plan = (ctypes.c_int * 6)()
     assert L.htr_linear_plan(m, n, K, M, nsplit, plan) == 0
-    assert plan[2] == (M + 95) // 96 and plan[1] == plan[3] * (m // 128) * plan[2]       # row tiles; splits x row blocks x tiles
+    heights = {3: (96,), 4: (128,), 0: (96, 128)}[T]
+    assert plan[2] in [-(-M // h) for h in heights] and plan[1] == plan[3] * (m // 128) * plan[2]   # row tiles; splits x row blocks x tiles
     if S:
         assert plan[3] == S
     need = L.htr_workspace_bytes(m, n, K, M, nsplit)
@@ -396,7 +400,7 @@ def test_more_than_128_rows_in_one_launch(dev, oracle, K, M, m, n, S):
     first = y.clone()
     ref = _ref(oracle, qw, sc, su, sv, x)
     got = first.cpu().numpy()
-    for r in (0, 95, 96, M // 2, M - 1):
+    for r in (0, 95, 96, 127, 128, M // 2, M - 1):
         if r < M:
             assert _rel(got[r], ref[r]) <= REL_TOL, (r, _rel(got[r], ref[r]))
     assert _rel(got, ref) <= REL_TOL
@@ -425,6 +429,7 @@ def test_fused_row_limit_follows_the_shape(dev, oracle, monkeypatch):
     from htr_amd import ops
     big = ops.ONE_LAUNCH
     assert ops.fused_max_rows(4096, 4096) == 384 and ops.fused_max_rows(14336, 4096) == 384 and ops.fused_max_rows(1024, 4096) == 128
+    assert ops.fused_max_rows(4096, 14336) == 512 and ops.fused_rows_per_launch(4096, 14336, 512) == big
     assert [ops.fused_rows_per_launch(14336, 4096, M) for M in (1, 128, 129, 384, 385)] == [128, 128, big, big, 0]
     assert [ops.fused_rows_per_launch(4096, 4096, M) for M in (129, 384, 385)] == [big, big, 0]
     assert ops.fused_rows_per_launch(2048, 2048, 129) == 0

@@ -113,23 +113,32 @@ def test_launch_plan_is_consistent(L, m, n, M):
 @pytest.mark.parametrize("m,n", [(128, 128), (4096, 4096), (14336, 4096), (4096, 14336), (28672, 4096)])
 @pytest.mark.parametrize("M", [129, 192, 193, 384, 1000, 2048])
 def test_plan_for_more_than_128_rows(L, m, n, M):
-    """The fused decode -> matrix-unit kernel: tiles of 96 activation rows, up to 8 column splits while the grid stays within
-    the compute units, no empty split; the workspace holds the rotated activations and, with splits, a tile per workgroup."""
+    """The fused decode -> matrix-unit kernel: tiles of 96 or 128 activation rows (the planner's choice; nsplit bits 20 / 21
+    force one), up to 4 column splits by policy (8 on request) while the grid stays within the compute units, no empty
+    split; the workspace holds the rotated activations and, with splits, a tile per workgroup."""
     out = (ctypes.c_int * 6)()
-    assert L.htr_linear_plan(m, n, 4, M, 0, out) == 0
-    cb, wgs, tiles, S, prerot, lds = list(out)
     nblk, rbs = n // 128, m // 128
-    assert tiles == -(-M // 96) and wgs == S * rbs * tiles and prerot == 1 and lds <= 160 * 1024
-    assert 1 <= S <= 8 and S == -(-nblk // cb) and (S == 1 or wgs <= 256)
-    need = L.htr_workspace_bytes(m, n, 4, M, 0)
-    assert need >= 256 + M * n * 2 + (wgs * 96 * 128 * 4 if S > 1 else 0)
+    for tile_bit, heights in ((0, (96, 128)), (1 << 20, (96,)), (1 << 21, (128,))):
+        ns = ((1 << 28) | tile_bit) if tile_bit else 0
+        assert L.htr_linear_plan(m, n, 4, M, ns, out) == 0
+        cb, wgs, tiles, S, prerot, lds = list(out)
+        rows = [h for h in heights if tiles == -(-M // h)]
+        assert rows and wgs == S * rbs * tiles and prerot == 1 and lds <= 160 * 1024
+        assert 1 <= S <= 4 and S == -(-nblk // cb) and (S == 1 or wgs <= 256)
+        need = L.htr_workspace_bytes(m, n, 4, M, ns)
+        assert need >= 256 + M * n * 2 + (wgs * rows[0] * 128 * 4 if S > 1 else 0)
     for want in (1, 2, 8):
+        ns = (1 << 28) | (1 << 20) | want
         if want > nblk or -(-nblk // -(-nblk // want)) != want:
-            assert L.htr_linear_plan(m, n, 4, M, (1 << 28) | want, out) != 0        # such a split would leave one empty
+            assert L.htr_linear_plan(m, n, 4, M, ns, out) != 0                      # such a split would leave one empty
             continue
-        assert L.htr_linear_plan(m, n, 4, M, (1 << 28) | want, out) == 0 and out[3] == want and out[1] == want * rbs * tiles
+        assert L.htr_linear_plan(m, n, 4, M, ns, out) == 0 and out[3] == want and out[1] == want * rbs * -(-M // 96)
     # bit 28 takes the kernel below its policy's row count too
     assert L.htr_linear_plan(m, n, 4, 40, (1 << 28) | 1, out) == 0 and out[2] == 1 and out[1] == rbs
+    # where a third 96-row tile would start a second round of workgroups, two 128-row tiles are taken
+    if (m, n, M) == (14336, 4096, 193):
+        assert L.htr_linear_plan(m, n, 4, 256, 0, out) == 0 and out[2] == 2 and out[1] == 224
+        assert L.htr_linear_plan(m, n, 4, 192, 0, out) == 0 and out[2] == 2 and out[5] == 101392
 
 
 @pytest.mark.parametrize("cus", [32, 64, 120, 256, 304])

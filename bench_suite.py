@@ -3,7 +3,7 @@ names (K x shape x batch table, 8..128 activation rows, routed experts, lm_head)
 
 Every case cycles through a ring of distinct weight copies larger than the caches (>= 1 GB, or as many copies as
 fit), replays the ring as one HIP graph and reads HIP events on the launch stream.  Used by `bench.py --suite`;
-`python bench_suite.py [names]` prints the same dictionary as JSON.
+`python bench_suite.py [names]` prints the same dictionary as JSON; `one:MxNxKxROWS` times a single shape.
 """
 import json
 import sys
@@ -233,12 +233,18 @@ CASES = {"table": table, "batch8_32": batch8_32, "moe": moe, "lm_head": lm_head,
 DEFAULT = ("table", "batch8_32", "moe", "lm_head")       # what bench.py reports by default: every baseline configuration
 
 
+def one(spec, dev):
+    """`one:MxNxKxROWS` - a single shape (for counter and trace runs of one kernel), e.g. one:14336x4096x4x192"""
+    m, n, K, M = (int(v) for v in spec.lower().split("x"))
+    return time_linear(m, n, K, M, dev)
+
+
 def run(names, dev=None):
     dev = dev or torch.device("cuda:0")
     names = list(CASES) if not names or "all" in names else [c for nm in names for c in (DEFAULT if nm == "default" else (nm,))]
     res = {}
     for nm in names:
-        res[nm] = CASES[nm](dev)
+        res[nm] = one(nm[4:], dev) if nm.startswith("one:") else CASES[nm](dev)
         torch.cuda.synchronize()
         torch.cuda.empty_cache()
     return res

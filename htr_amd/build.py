@@ -10,7 +10,9 @@ import sys
 
 CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 LIB = os.path.join(CSRC, "libhtr_gfx950.so")
-SOURCES = [os.path.join(CSRC, "htr_gfx950.hip")]
+SOURCES = [os.path.join(CSRC, "htr_gfx950.hip")]          # one translation unit; the kernels live in the parts it includes
+PARTS = [os.path.join(CSRC, f) for f in ("decode.hpp", "linear.hpp", "linear_batch.hpp", "linear_gemm.hpp", "dequant.hpp",
+                                         "viterbi.hpp", "anchors.hpp", "plan.hpp")]
 HEADER = os.path.join(os.path.dirname(CSRC), os.pardir, "include", "htr_gfx950.h")
 
 HIPCC_FLAGS = [
@@ -42,7 +44,7 @@ def is_stale():
     if not os.path.exists(LIB):
         return True
     t = os.path.getmtime(LIB)
-    return any(os.path.getmtime(s) > t for s in SOURCES + [HEADER])
+    return any(os.path.getmtime(s) > t for s in SOURCES + PARTS + [HEADER])
 
 
 if __name__ == "__main__":
